@@ -1,0 +1,164 @@
+/*
+ * libptj -- C ABI of the MI355X (gfx950) kernel path that replaces the Triton
+ * kernels of martin-kukla/pre-tjax (model_triton.py, loss_and_optimizer_triton.py).
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless said
+ *     otherwise; the caller owns all buffers (inputs, outputs, workspaces);
+ *   - no entry point allocates, frees or synchronises; work is enqueued on
+ *     `stream` (a hipStream_t passed as void*, NULL = the default stream);
+ *   - `dtype` selects the storage type of all float tensors of the call
+ *     (PTJ_F32 or PTJ_BF16); statistics and accumulators are always fp32;
+ *   - strides are in ELEMENTS;
+ *   - return value 0 on success, negative PTJ_ERR_* otherwise, in which case
+ *     ptj_last_error() (thread local) describes the failure.  Nothing is launched
+ *     when an argument check fails.
+ * The reference interface each entry point replaces is cited as
+ * `model_triton.py:<line>` (kernel / wrapper) relative to the reference tree.
+ */
+#ifndef PTJ_H
+#define PTJ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTJ_F32 0
+#define PTJ_BF16 1
+
+#define PTJ_OK 0
+#define PTJ_ERR_INVALID (-1)     /* bad argument / unsupported shape */
+#define PTJ_ERR_LAUNCH (-2)      /* HIP reported a launch error */
+#define PTJ_ERR_WORKSPACE (-3)   /* workspace too small */
+
+/* GEMM epilogues (ptj_gemm) */
+#define PTJ_EPI_NONE 0
+#define PTJ_EPI_BIAS 1           /* C = A.B + bias[m]                       */
+#define PTJ_EPI_BIAS_GELU 2      /* C = gelu(A.B + bias[m])                 */
+
+int ptj_version(void);
+const char* ptj_last_error(void);
+
+/* ---- row-wise kernels ---------------------------------------------------- */
+
+/* LayerNorm forward: y = gamma*(x-mean)/std_unbiased + beta, no epsilon.
+ * Replaces t_layernorm_fwd_k / t_layernorm_fwd_t (model_triton.py:1582-1637). */
+int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y,
+                      int64_t rows, int64_t cols, int64_t x_row_stride, int64_t y_row_stride,
+                      int dtype, void* stream);
+
+/* LayerNorm backward.  dx (nullable) replaces t_layernorm_bkwd2_x_k/_t
+ * (model_triton.py:1799-1867); dgamma/dbeta (both nullable together) replace
+ * t_layernorm_bkwd2_p_k/_t (model_triton.py:1664-1726) with a deterministic
+ * two-stage reduction instead of float atomics.  `workspace` must hold
+ * ptj_layernorm_bwd_workspace_bytes(rows, cols) bytes when dgamma != NULL
+ * (may be NULL otherwise).  gamma may be NULL when dx == NULL. */
+size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols);
+int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma,
+                      void* dx, void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes,
+                      int64_t rows, int64_t cols, int64_t dy_row_stride, int64_t x_row_stride,
+                      int64_t dx_row_stride, int dtype, void* stream);
+
+/* tanh-GELU forward / backward on a flat array of n elements.
+ * Replace t_gelu_fwd_k/_t (model_triton.py:237-260) and t_gelu_bkwd2_k/_t (:274-304). */
+int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
+int ptj_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype, void* stream);
+
+/* Dropout, rate 0.1, non-inverted: train != 0 -> y = keep ? x : 0 with
+ * keep = tl.rand(seed + row, col) > 0.1 (Philox4x32-10); train == 0 -> y = 0.9*x.
+ * The backward applies the same function to dy, so one entry point serves
+ * t_dropout_fwd_k/_t (model_triton.py:1471-1506) and t_dropout_bkwd2_k/_t (:1538-1572). */
+int ptj_dropout(const void* x, void* y, int64_t rows, int64_t cols,
+                int64_t x_row_stride, int64_t y_row_stride,
+                int train, int64_t seed, int dtype, void* stream);
+
+/* Fused residual update used by the block composites: y = res + dropout(x) with
+ * the same mask as ptj_dropout (model_triton.py:1898, 2069: y + t_dropout_fwd_t(...)).
+ * All three tensors are contiguous [rows, cols]. */
+int ptj_dropout_add(const void* x, const void* res, void* y, int64_t rows, int64_t cols,
+                    int train, int64_t seed, int dtype, void* stream);
+
+/* Row-wise log-softmax forward / backward (dx = dy - softmax(x)*sum(dy)).
+ * Replace t_log_softmax_fwd_k/_t (model_triton.py:30-72) and
+ * t_log_softmax_bkwd2_k/_t (:122-164). */
+int ptj_log_softmax_fwd(const void* x, void* y, int64_t rows, int64_t cols,
+                        int64_t x_row_stride, int64_t y_row_stride, int dtype, void* stream);
+int ptj_log_softmax_bwd(const void* dy, const void* x, void* dx, int64_t rows, int64_t cols,
+                        int64_t dy_row_stride, int64_t x_row_stride, int64_t dx_row_stride,
+                        int dtype, void* stream);
+
+/* Fused log-softmax + mean cross-entropy forward and backward over rows whose
+ * label != 0.  Replaces t_avg_cross_entropy_loss_bkwd3_k/_t
+ * (loss_and_optimizer_triton.py:108-197).
+ *   labels  int64 [rows];  logits/dlogits [rows, cols] with row strides;
+ *   loss    float [1]  (fp32 regardless of dtype) = -mean_{label!=0} log_softmax(x)[label];
+ *   count   int64 [1]  = number of labels != 0;
+ *   dlogits = (softmax(x) - onehot(label))/count on rows with label != 0, else 0.
+ * dlogits may alias logits (in-place).  `workspace`: ptj_ce_workspace_bytes(rows) bytes.
+ * Deterministic (no atomics).  count == 0 gives loss = NaN as the reference does. */
+size_t ptj_ce_workspace_bytes(int64_t rows);
+int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64_t* count,
+                   void* dlogits, void* workspace, size_t workspace_bytes,
+                   int64_t rows, int64_t cols, int64_t logits_row_stride, int64_t dlogits_row_stride,
+                   int dtype, void* stream);
+
+/* ---- dense contraction --------------------------------------------------- */
+
+/* C[n,m] = sum_k A(n,k) * B(k,m) (+ bias[m]) (gelu) with fp32 accumulation on MFMA.
+ * A(n,k) = a[n*a_rs + k*a_cs], B(k,m) = b[k*b_rs + m*b_cs]; for each operand one
+ * of the two strides must be 1 (row- or column-major views, as produced by
+ * `.t()`), C is row-major with row stride c_rs.  Replaces t_matmul_k / t_matmul_t
+ * (model_triton.py:313-398) and the two launches of t_tlayer_ffn_fwd_t (:1258-1313);
+ * also the torch.matmul / einsum call sites of the training path
+ * (:306, :436, :460-472, :495-508, :423-428). */
+int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
+             int64_t n, int64_t m, int64_t k,
+             int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs,
+             int epilogue, int dtype, void* stream);
+
+/* ---- attention ----------------------------------------------------------- */
+
+/* Causal flash-attention forward.  q/k/v/o are [BH, T, dh] views with explicit
+ * (batch-head, row) strides and unit stride along dh; `mask` is NULL (pure causal:
+ * key j visible to query i iff j <= i) or uint8 [B, T, T] (contiguous) that is
+ * ANDed with the causal block structure exactly as the reference kernel does
+ * (tiles strictly above the diagonal are never visited; model_triton.py:659-661).
+ * Saves ms (running row max of the scaled, masked scores) and ls (sum of
+ * exp(score - ms)) as fp32 [BH, T].  Dropout (train != 0) keeps probability
+ * (i, j) of batch-head g iff tl.rand(seed + g, i + j) > 0.1; train == 0 scales
+ * probabilities by 0.9.  Replaces t_scaled_dot_prod_attn_fwd3_k/_t
+ * (model_triton.py:616-754).  Requires dh == 64 and T % 64 == 0. */
+int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mask,
+                 void* o, float* ms, float* ls,
+                 int64_t B, int64_t H, int64_t T, int64_t dh,
+                 int64_t q_bh_stride, int64_t q_row_stride,
+                 int64_t k_bh_stride, int64_t k_row_stride,
+                 int64_t v_bh_stride, int64_t v_row_stride,
+                 int64_t o_bh_stride, int64_t o_row_stride,
+                 int train, int64_t seed, int dtype, void* stream);
+
+/* Flash-attention backward with P recomputed from (ms, ls).  Outputs dq/dk/dv
+ * [BH, T, dh] with explicit strides.  Deterministic: dK/dV and dQ are produced by
+ * two passes, no atomics.  Replaces t_scaled_dot_prod_attn_bkwd3_k/_t
+ * (model_triton.py:829-1003). */
+int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o,
+                 const float* ms, const float* ls, const uint8_t* mask,
+                 void* dq, void* dk, void* dv,
+                 int64_t B, int64_t H, int64_t T, int64_t dh,
+                 int64_t do_bh_stride, int64_t do_row_stride,
+                 int64_t q_bh_stride, int64_t q_row_stride,
+                 int64_t k_bh_stride, int64_t k_row_stride,
+                 int64_t v_bh_stride, int64_t v_row_stride,
+                 int64_t o_bh_stride, int64_t o_row_stride,
+                 int64_t dq_bh_stride, int64_t dq_row_stride,
+                 int64_t dk_bh_stride, int64_t dk_row_stride,
+                 int64_t dv_bh_stride, int64_t dv_row_stride,
+                 int train, int64_t seed, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTJ_H */

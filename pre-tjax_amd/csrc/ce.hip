@@ -1,0 +1,223 @@
+// Fused log-softmax + mean cross-entropy, forward and backward in one pass over the
+// logits: each row (vocabulary-wide, e.g. 50257) is read from HBM once into the
+// registers of a 1024-thread workgroup, reduced (max, sum-exp), and the gradient row
+// is written once.  Rows are not 16-byte aligned when the vocabulary size is odd, so
+// vectors are taken relative to the aligned address below the row start and the two
+// boundary vectors of a row are masked element-wise.
+#include "common.h"
+
+namespace {
+
+constexpr int CE_THREADS = 1024;
+
+__global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restrict__ labels, int64_t rows,
+                                                         int64_t* __restrict__ count) {
+    __shared__ int sm[16];
+    int c = 0;
+    for (int64_t i = threadIdx.x; i < rows; i += 1024) c += labels[i] != 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int64_t t = 0;
+        for (int i = 0; i < 16; ++i) t += sm[i];
+        *count = t;
+    }
+}
+
+// CACHED: the row is kept in registers (ITERS vectors per thread).  Otherwise the
+// row is streamed from memory three times (max, sum, gradient).
+template <typename T, int ITERS, bool CACHED>
+__global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict__ labels, const T* logits,
+                                                       T* dlogits, float* __restrict__ row_loss,
+                                                       const int64_t* __restrict__ count, int64_t rows, int cols,
+                                                       int64_t xs, int64_t dxs) {
+    constexpr int VEC = VecOf<T>::N;
+    __shared__ float smem[16];
+    __shared__ float s_xy;
+    const int t = threadIdx.x;
+    const float inv_cnt = 1.0f / (float)(*count);
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const T* xr = logits + row * xs;
+        T* dr = dlogits + row * dxs;
+        const int mis = (int)((reinterpret_cast<uintptr_t>(xr) & 15) / sizeof(T));
+        const T* xb = xr - mis;  // 16-byte aligned
+        T* db = dr - mis;        // 16-byte aligned too (checked on the host)
+        const int nvec = (cols + mis + VEC - 1) / VEC;
+        const int64_t label = labels[row];
+        if (t == 0 && label != 0) s_xy = to_f32(xr[label]);  // read before any in-place write
+
+        float v[ITERS][VEC];
+        float m = -INFINITY;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int vi = t + it * CE_THREADS;
+                if (vi < nvec) {
+                    load_vec<T, VEC>(xb + (int64_t)vi * VEC, v[it]);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const int e = vi * VEC + j - mis;
+                        if (e < 0 || e >= cols) v[it][j] = -INFINITY;
+                        m = fmaxf(m, v[it][j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) v[it][j] = -INFINITY;
+                }
+            }
+        } else {
+            for (int vi = t; vi < nvec; vi += CE_THREADS) {
+                float w[VEC];
+                load_vec<T, VEC>(xb + (int64_t)vi * VEC, w);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int e = vi * VEC + j - mis;
+                    if (e >= 0 && e < cols) m = fmaxf(m, w[j]);
+                }
+            }
+        }
+        m = row_reduce<CE_THREADS, true>(m, smem);
+        float s = 0.f;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    v[it][j] = __expf(v[it][j] - m);
+                    s += v[it][j];
+                }
+        } else {
+            for (int vi = t; vi < nvec; vi += CE_THREADS) {
+                float w[VEC];
+                load_vec<T, VEC>(xb + (int64_t)vi * VEC, w);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int e = vi * VEC + j - mis;
+                    if (e >= 0 && e < cols) s += __expf(w[j] - m);
+                }
+            }
+        }
+        s = row_reduce<CE_THREADS, false>(s, smem);  // contains __syncthreads: s_xy is visible after it
+        const bool live = label != 0;
+        if (t == 0) row_loss[row] = live ? -(s_xy - m - logf(s)) : 0.f;
+        const float scale = live ? inv_cnt / s : 0.f;
+
+        auto emit = [&](int vi, float (&g)[VEC]) {
+            const int e0 = vi * VEC - mis;
+            if (live) {
+                const int64_t lj = label - e0;
+                if (lj >= 0 && lj < VEC) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (j == (int)lj) g[j] -= inv_cnt;
+                }
+            }
+            if (e0 >= 0 && e0 + VEC <= cols) {
+                store_vec<T, VEC>(db + (int64_t)vi * VEC, g);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int e = e0 + j;
+                    if (e >= 0 && e < cols) dr[e] = from_f32<T>(g[j]);
+                }
+            }
+        };
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int vi = t + it * CE_THREADS;
+                if (vi < nvec) {
+                    float g[VEC];
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) g[j] = v[it][j] * scale;
+                    emit(vi, g);
+                }
+            }
+        } else {
+            for (int vi = t; vi < nvec; vi += CE_THREADS) {
+                float g[VEC];
+                load_vec<T, VEC>(xb + (int64_t)vi * VEC, g);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) g[j] = __expf(g[j] - m) * scale;
+                emit(vi, g);
+            }
+        }
+        __syncthreads();  // s_xy is rewritten by thread 0 at the top of the next row
+    }
+}
+
+// loss = (sum of row losses in index order) / count.  One workgroup, fixed order.
+__global__ __launch_bounds__(1024) void ce_finalize_kernel(const float* __restrict__ row_loss, int64_t rows,
+                                                            const int64_t* __restrict__ count,
+                                                            float* __restrict__ loss) {
+    __shared__ float sm[1024];
+    // Each thread sums a contiguous slice so the summation order is fixed.
+    const int64_t per = (rows + 1023) / 1024;
+    const int64_t b = threadIdx.x * per;
+    const int64_t e = b + per < rows ? b + per : rows;
+    float s = 0.f;
+    for (int64_t i = b; i < e; ++i) s += row_loss[i];
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = 512; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) sm[threadIdx.x] += sm[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss = sm[0] / (float)(*count);
+}
+
+template <typename T>
+int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits, void* ws,
+            int64_t rows, int64_t cols, int64_t xs, int64_t dxs, hipStream_t st) {
+    constexpr int VEC = VecOf<T>::N;
+    constexpr int ITERS = 64 / VEC;  // 64 cached floats per thread
+    float* row_loss = (float*)ws;
+    hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows, count);
+    PTJ_CHECK_LAUNCH();
+    const int grid = (int)(rows < 256 * 2 ? rows : 256 * 2);
+    const bool cached = (cols + VEC) <= (int64_t)CE_THREADS * ITERS * VEC;
+    if (cached)
+        hipLaunchKernelGGL((ce_row_kernel<T, ITERS, true>), dim3(grid), dim3(1024), 0, st, labels, (const T*)logits,
+                           (T*)dlogits, row_loss, (const int64_t*)count, rows, (int)cols, xs, dxs);
+    else
+        hipLaunchKernelGGL((ce_row_kernel<T, 1, false>), dim3(grid), dim3(1024), 0, st, labels, (const T*)logits,
+                           (T*)dlogits, row_loss, (const int64_t*)count, rows, (int)cols, xs, dxs);
+    PTJ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)row_loss, rows,
+                       (const int64_t*)count, loss);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t ptj_ce_workspace_bytes(int64_t rows) { return rows > 0 ? (size_t)rows * sizeof(float) : 0; }
+
+int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
+                   void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t xs, int64_t dxs,
+                   int dtype, void* stream) {
+    PTJ_CHECK_ARG(labels && logits && loss && count && dlogits, "ce_fwd_bwd: null pointer");
+    PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 30), "ce_fwd_bwd: bad shape %lld x %lld", (long long)rows,
+                  (long long)cols);
+    PTJ_CHECK_ARG(xs >= cols && dxs >= cols, "ce_fwd_bwd: row stride smaller than cols");
+    if (!workspace || workspace_bytes < ptj_ce_workspace_bytes(rows))
+        return ptj_set_error(PTJ_ERR_WORKSPACE, "ce_fwd_bwd: workspace %zu < %zu bytes", workspace_bytes,
+                             ptj_ce_workspace_bytes(rows));
+    const size_t es = dtype == PTJ_BF16 ? 2 : 4;
+    // Every gradient row must share its logits row's offset inside a 16-byte line.
+    PTJ_CHECK_ARG(((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(dlogits)) & 15) == 0 &&
+                      (((xs - dxs) * (int64_t)es) % 16 == 0 || rows == 1),
+                  "ce_fwd_bwd: logits and dlogits rows must have equal 16-byte misalignment");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case PTJ_F32: return ce_impl<float>(labels, logits, loss, count, dlogits, workspace, rows, cols, xs, dxs, st);
+        case PTJ_BF16: return ce_impl<bf16>(labels, logits, loss, count, dlogits, workspace, rows, cols, xs, dxs, st);
+        default: return ptj_set_error(PTJ_ERR_INVALID, "ce_fwd_bwd: unknown dtype %d", dtype);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,645 @@
+// Row-wise, HBM-bound kernels: LayerNorm fwd/bwd, tanh-GELU fwd/bwd, Philox dropout,
+// log-softmax fwd/bwd.  One row is owned by TPR threads (one wavefront for short rows,
+// a 256- or 1024-thread workgroup for long ones) and lives in registers between the
+// single HBM read and the single HBM write; all global accesses are 16-byte vectors
+// when shapes allow (VEC = 16/sizeof(T)), scalar otherwise.
+#include "common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------
+// Row holder: thread `t` of the TPR threads owning a row holds vectors
+// t, t+TPR, t+2*TPR, ... (ITERS of them), each VEC consecutive elements.
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC, int TPR, int ITERS>
+struct RowRegs {
+    float v[ITERS][VEC];
+    __device__ __forceinline__ void load(const T* __restrict__ row, int nvec, int t, float fill) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int vi = t + it * TPR;
+            if (vi < nvec) {
+                load_vec<T, VEC>(row + (int64_t)vi * VEC, v[it]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[it][j] = fill;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(T* __restrict__ row, int nvec, int t) const {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int vi = t + it * TPR;
+            if (vi < nvec) store_vec<T, VEC>(row + (int64_t)vi * VEC, v[it]);
+        }
+    }
+};
+
+template <int TPR> struct RowGeom {
+    static constexpr int BLOCK = TPR == 64 ? 256 : TPR;
+    static constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
+};
+
+// ---------------------------------------------------------------------------------
+// LayerNorm forward
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC, int TPR, int ITERS>
+__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ y,
+    int64_t rows, int cols, int64_t xs, int64_t ys) {
+    __shared__ float smem[16];
+    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    const int t = threadIdx.x % TPR;
+    const int sub = threadIdx.x / TPR;
+    const int nvec = cols / VEC;
+    RowRegs<T, VEC, TPR, ITERS> g, b;
+    g.load(gamma, nvec, t, 0.f);
+    b.load(beta, nvec, t, 0.f);
+    const float inv_n = 1.0f / (float)cols;
+    const float inv_nm1 = 1.0f / (float)(cols - 1);
+    for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
+        RowRegs<T, VEC, TPR, ITERS> r;
+        r.load(x + row * xs, nvec, t, 0.f);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += r.v[it][j];
+        const float mu = row_reduce<TPR, false>(s, smem) * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const bool valid = (t + it * TPR) < nvec;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float d = valid ? r.v[it][j] - mu : 0.f;
+                r.v[it][j] = d;
+                q += d * d;
+            }
+        }
+        const float var = row_reduce<TPR, false>(q, smem) * inv_nm1;
+        const float rstd = 1.0f / sqrtf(var);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[it][j] = g.v[it][j] * (r.v[it][j] * rstd) + b.v[it][j];
+        r.store(y + row * ys, nvec, t);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// LayerNorm backward: dx and/or per-block partial sums of dgamma, dbeta.
+// Partials layout: part[p][0][cols] = sum dy*xhat, part[p][1][cols] = sum dy over the
+// rows handled by row-slot p (p = blockIdx.x*RPB + sub).
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
+__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, T* __restrict__ dx,
+    float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs) {
+    __shared__ float smem[16];
+    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    const int t = threadIdx.x % TPR;
+    const int sub = threadIdx.x / TPR;
+    const int nvec = cols / VEC;
+    RowRegs<T, VEC, TPR, ITERS> g;
+    if constexpr (DX) g.load(gamma, nvec, t, 0.f);
+    float acc_g[ITERS][VEC], acc_b[ITERS][VEC];
+    if constexpr (DGB) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc_g[it][j] = acc_b[it][j] = 0.f;
+    }
+    const float inv_n = 1.0f / (float)cols;
+    const float inv_nm1 = 1.0f / (float)(cols - 1);
+    const float n_adj = (float)cols * inv_nm1;
+    // Every thread of a >64-thread row group must take the same trip count because
+    // row_reduce synchronises the block; with RPB == 1 all threads share `row`.
+    for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
+        RowRegs<T, VEC, TPR, ITERS> r, d;
+        r.load(x + row * xs, nvec, t, 0.f);
+        d.load(dy + row * dys, nvec, t, 0.f);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += r.v[it][j];
+        const float mu = row_reduce<TPR, false>(s, smem) * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const bool valid = (t + it * TPR) < nvec;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float c = valid ? r.v[it][j] - mu : 0.f;
+                r.v[it][j] = c;
+                q += c * c;
+            }
+        }
+        const float var = row_reduce<TPR, false>(q, smem) * inv_nm1;
+        const float rstd = 1.0f / sqrtf(var);
+        float sg = 0.f, sgx = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xh = r.v[it][j] * rstd;
+                r.v[it][j] = xh;
+                if constexpr (DGB) {
+                    acc_g[it][j] += d.v[it][j] * xh;
+                    acc_b[it][j] += d.v[it][j];
+                }
+                if constexpr (DX) {
+                    const float gg = d.v[it][j] * g.v[it][j];
+                    d.v[it][j] = gg;
+                    sg += gg;
+                    sgx += gg * xh;
+                }
+            }
+        if constexpr (DX) {
+            const float mg = row_reduce<TPR, false>(sg, smem) * inv_n;
+            const float mgx = row_reduce<TPR, false>(sgx, smem) * inv_n * n_adj;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) d.v[it][j] = (d.v[it][j] - mg - r.v[it][j] * mgx) * rstd;
+            d.store(dx + row * dxs, nvec, t);
+        }
+    }
+    if constexpr (DGB) {
+        const int64_t p = (int64_t)blockIdx.x * RPB + sub;
+        float* pg = part + p * 2 * (int64_t)cols;
+        float* pb = pg + cols;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int vi = t + it * TPR;
+            if (vi < nvec) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    pg[vi * VEC + j] = acc_g[it][j];
+                    pb[vi * VEC + j] = acc_b[it][j];
+                }
+            }
+        }
+    }
+}
+
+// Second stage: out[which][c] = sum_p part[p][which][c], fixed order.
+// Block = 256 threads = 32 columns x 8 partial-slices; grid = (ceil(cols/32), 2).
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float* __restrict__ part, int nparts,
+                                                                    int cols, T* __restrict__ dgamma,
+                                                                    T* __restrict__ dbeta) {
+    __shared__ float sm[8][33];
+    const int cx = threadIdx.x & 31, py = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + cx;
+    const int which = blockIdx.y;
+    float s = 0.f;
+    if (c < cols)
+        for (int p = py; p < nparts; p += 8) s += part[((int64_t)p * 2 + which) * cols + c];
+    sm[py][cx] = s;
+    __syncthreads();
+    if (py == 0 && c < cols) {
+        float r = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r += sm[i][cx];
+        (which == 0 ? dgamma : dbeta)[c] = from_f32<T>(r);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// log-softmax forward / backward
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC, int TPR, int ITERS>
+__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void log_softmax_fwd_kernel(const T* __restrict__ x,
+                                                                               T* __restrict__ y, int64_t rows,
+                                                                               int cols, int64_t xs, int64_t ys) {
+    __shared__ float smem[16];
+    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    const int t = threadIdx.x % TPR;
+    const int sub = threadIdx.x / TPR;
+    const int nvec = cols / VEC;
+    for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
+        RowRegs<T, VEC, TPR, ITERS> r;
+        r.load(x + row * xs, nvec, t, -INFINITY);
+        float m = -INFINITY;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) m = fmaxf(m, r.v[it][j]);
+        m = row_reduce<TPR, true>(m, smem);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                r.v[it][j] -= m;
+                s += __expf(r.v[it][j]);
+            }
+        const float lse = logf(row_reduce<TPR, false>(s, smem));
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[it][j] -= lse;
+        r.store(y + row * ys, nvec, t);
+    }
+}
+
+template <typename T, int VEC, int TPR, int ITERS>
+__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void log_softmax_bwd_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, T* __restrict__ dx, int64_t rows, int cols, int64_t dys,
+    int64_t xs, int64_t dxs) {
+    __shared__ float smem[16];
+    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    const int t = threadIdx.x % TPR;
+    const int sub = threadIdx.x / TPR;
+    const int nvec = cols / VEC;
+    for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
+        RowRegs<T, VEC, TPR, ITERS> r, d;
+        r.load(x + row * xs, nvec, t, -INFINITY);
+        d.load(dy + row * dys, nvec, t, 0.f);
+        float m = -INFINITY, sd = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                m = fmaxf(m, r.v[it][j]);
+                sd += d.v[it][j];
+            }
+        m = row_reduce<TPR, true>(m, smem);
+        sd = row_reduce<TPR, false>(sd, smem);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                r.v[it][j] = __expf(r.v[it][j] - m);
+                s += r.v[it][j];
+            }
+        const float c = sd / row_reduce<TPR, false>(s, smem);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) d.v[it][j] -= r.v[it][j] * c;
+        d.store(dx + row * dxs, nvec, t);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Elementwise: GELU fwd/bwd (flat), dropout (+ residual add)
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gelu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t nvec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float v[VEC];
+        load_vec<T, VEC>(x + i * VEC, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = gelu_f(v[j]);
+        store_vec<T, VEC>(y + i * VEC, v);
+    }
+}
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gelu_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                        T* __restrict__ dx, int64_t nvec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float v[VEC], d[VEC];
+        load_vec<T, VEC>(x + i * VEC, v);
+        load_vec<T, VEC>(dy + i * VEC, d);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) d[j] *= gelu_grad_f(v[j]);
+        store_vec<T, VEC>(dx + i * VEC, d);
+    }
+}
+
+// One thread per VEC-wide chunk; chunks never straddle rows (cols % VEC == 0).
+template <typename T, int VEC, bool ADD>
+__global__ __launch_bounds__(256) void dropout_kernel(const T* __restrict__ x, const T* __restrict__ res,
+                                                       T* __restrict__ y, int64_t rows, int cols, int64_t xs,
+                                                       int64_t ys, int train, uint64_t seed) {
+    const int vpr = cols / VEC;  // vectors per row
+    const int64_t total = rows * vpr;
+    const bool small = total <= 0x7fffffffll;  // 32-bit division is several times cheaper
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = small ? (int64_t)((uint32_t)i / (uint32_t)vpr) : i / vpr;
+        const int c0 = (int)(i - row * vpr) * VEC;
+        float v[VEC];
+        load_vec<T, VEC>(x + row * xs + c0, v);
+        if (train) {
+            const uint64_t s = seed + (uint64_t)row;
+            const uint32_t k0 = (uint32_t)s, k1 = (uint32_t)(s >> 32);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = philox_keep((uint32_t)(c0 + j), k0, k1) ? v[j] : 0.f;
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= 0.9f;
+        }
+        if constexpr (ADD) {
+            float r[VEC];
+            load_vec<T, VEC>(res + row * (int64_t)cols + c0, r);
+            // The reference rounds dropout(x) to the storage type before adding it.
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = r[j] + to_f32(from_f32<T>(v[j]));
+        }
+        store_vec<T, VEC>(y + row * ys + c0, v);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Dispatch helpers
+// ---------------------------------------------------------------------------------
+struct RowCfg {
+    int vec;   // VEC or 1
+    int tpr;   // 64, 256, 1024
+};
+
+// Picks the smallest row-group that holds `cols` elements in registers.
+// ITERS is fixed per TPR: 64 -> 4, 256 -> 4, 1024 -> 8.
+inline bool pick_row_cfg(int64_t cols, int full_vec, bool vec_ok, RowCfg* cfg) {
+    const int vec = vec_ok ? full_vec : 1;
+    const int64_t nvec = cols / vec;
+    cfg->vec = vec;
+    if (nvec <= 64 * 4) cfg->tpr = 64;
+    else if (nvec <= 256 * 4) cfg->tpr = 256;
+    else if (nvec <= 1024 * 8) cfg->tpr = 1024;
+    else return false;
+    return true;
+}
+
+inline int row_grid(int64_t rows, int tpr) {
+    const int rpb = tpr == 64 ? 4 : 1;
+    const int64_t need = (rows + rpb - 1) / rpb;
+    const int64_t cap = 256 * 8;  // 8 workgroups per CU on 256 CUs
+    return (int)(need < cap ? need : cap);
+}
+
+#define ROW_DISPATCH(T, cfg, LAUNCH)                                     \
+    do {                                                                 \
+        constexpr int FV = VecOf<T>::N;                                  \
+        if (cfg.vec == 1) {                                              \
+            if (cfg.tpr == 64) { LAUNCH(T, 1, 64, 4); }                  \
+            else if (cfg.tpr == 256) { LAUNCH(T, 1, 256, 4); }           \
+            else { LAUNCH(T, 1, 1024, 8); }                              \
+        } else {                                                         \
+            if (cfg.tpr == 64) { LAUNCH(T, FV, 64, 4); }                 \
+            else if (cfg.tpr == 256) { LAUNCH(T, FV, 256, 4); }          \
+            else { LAUNCH(T, FV, 1024, 8); }                             \
+        }                                                                \
+    } while (0)
+
+template <typename T>
+bool rows_vec_ok(int64_t cols, std::initializer_list<const void*> ptrs, std::initializer_list<int64_t> strides) {
+    constexpr int FV = VecOf<T>::N;
+    if (cols % FV) return false;
+    for (const void* p : ptrs)
+        if (p && !ptj_aligned16(p)) return false;
+    for (int64_t s : strides)
+        if (s % FV) return false;
+    return true;
+}
+
+template <typename T>
+int layernorm_fwd_impl(const void* x, const void* gamma, const void* beta, void* y, int64_t rows, int64_t cols,
+                       int64_t xs, int64_t ys, hipStream_t st) {
+    RowCfg cfg;
+    const bool vok = rows_vec_ok<T>(cols, {x, gamma, beta, y}, {xs, ys});
+    if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
+        return ptj_set_error(PTJ_ERR_INVALID, "layernorm_fwd: cols=%lld too large for the register-resident row kernel",
+                             (long long)cols);
+    const int grid = row_grid(rows, cfg.tpr);
+#define LAUNCH(T_, V_, TPR_, IT_)                                                                           \
+    hipLaunchKernelGGL((layernorm_fwd_kernel<T_, V_, TPR_, IT_>), dim3(grid), dim3(RowGeom<TPR_>::BLOCK), 0, st, \
+                       (const T_*)x, (const T_*)gamma, (const T_*)beta, (T_*)y, rows, (int)cols, xs, ys)
+    ROW_DISPATCH(T, cfg, LAUNCH);
+#undef LAUNCH
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+inline int ln_bwd_nparts(int64_t rows, int tpr) { return row_grid(rows, tpr) * (tpr == 64 ? 4 : 1); }
+
+template <typename T>
+int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
+                       void* ws, size_t ws_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs, int64_t dxs,
+                       hipStream_t st) {
+    RowCfg cfg;
+    const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx}, {dys, xs, dx ? dxs : 0});
+    if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
+        return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: cols=%lld too large", (long long)cols);
+    const int grid = row_grid(rows, cfg.tpr);
+    const int nparts = ln_bwd_nparts(rows, cfg.tpr);
+    const bool want_dx = dx != nullptr, want_dgb = dgamma != nullptr;
+    if (want_dgb) {
+        const size_t need = (size_t)nparts * 2 * (size_t)cols * sizeof(float);
+        if (!ws || ws_bytes < need)
+            return ptj_set_error(PTJ_ERR_WORKSPACE, "layernorm_bwd: workspace %zu < %zu bytes", ws_bytes, need);
+    }
+#define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_)                                                                   \
+    hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
+                       dim3(RowGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (T_*)dx, \
+                       (float*)ws, rows, (int)cols, dys, xs, dxs)
+#define LAUNCH(T_, V_, TPR_, IT_)                                     \
+    do {                                                              \
+        if (want_dx && want_dgb) LAUNCH_F(T_, V_, TPR_, IT_, true, true);   \
+        else if (want_dx) LAUNCH_F(T_, V_, TPR_, IT_, true, false);   \
+        else LAUNCH_F(T_, V_, TPR_, IT_, false, true);                \
+    } while (0)
+    ROW_DISPATCH(T, cfg, LAUNCH);
+#undef LAUNCH
+#undef LAUNCH_F
+    PTJ_CHECK_LAUNCH();
+    if (want_dgb) {
+        hipLaunchKernelGGL((layernorm_bwd_reduce_kernel<T>), dim3((unsigned)((cols + 31) / 32), 2), dim3(256), 0, st,
+                           (const float*)ws, nparts, (int)cols, (T*)dgamma, (T*)dbeta);
+        PTJ_CHECK_LAUNCH();
+    }
+    return PTJ_OK;
+}
+
+template <typename T>
+int log_softmax_fwd_impl(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, hipStream_t st) {
+    RowCfg cfg;
+    const bool vok = rows_vec_ok<T>(cols, {x, y}, {xs, ys});
+    if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
+        return ptj_set_error(PTJ_ERR_INVALID, "log_softmax_fwd: cols=%lld too large", (long long)cols);
+    const int grid = row_grid(rows, cfg.tpr);
+#define LAUNCH(T_, V_, TPR_, IT_)                                                                              \
+    hipLaunchKernelGGL((log_softmax_fwd_kernel<T_, V_, TPR_, IT_>), dim3(grid), dim3(RowGeom<TPR_>::BLOCK), 0, st, \
+                       (const T_*)x, (T_*)y, rows, (int)cols, xs, ys)
+    ROW_DISPATCH(T, cfg, LAUNCH);
+#undef LAUNCH
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+template <typename T>
+int log_softmax_bwd_impl(const void* dy, const void* x, void* dx, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
+                         int64_t dxs, hipStream_t st) {
+    RowCfg cfg;
+    const bool vok = rows_vec_ok<T>(cols, {dy, x, dx}, {dys, xs, dxs});
+    if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
+        return ptj_set_error(PTJ_ERR_INVALID, "log_softmax_bwd: cols=%lld too large", (long long)cols);
+    const int grid = row_grid(rows, cfg.tpr);
+#define LAUNCH(T_, V_, TPR_, IT_)                                                                              \
+    hipLaunchKernelGGL((log_softmax_bwd_kernel<T_, V_, TPR_, IT_>), dim3(grid), dim3(RowGeom<TPR_>::BLOCK), 0, st, \
+                       (const T_*)dy, (const T_*)x, (T_*)dx, rows, (int)cols, dys, xs, dxs)
+    ROW_DISPATCH(T, cfg, LAUNCH);
+#undef LAUNCH
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+inline int flat_grid(int64_t nthreads_needed) {
+    int64_t b = (nthreads_needed + 255) / 256;
+    const int64_t cap = 256 * 16;
+    if (b > cap) b = cap;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+template <typename T>
+int gelu_impl(const void* dy, const void* x, void* out, int64_t n, bool bwd, hipStream_t st) {
+    constexpr int FV = VecOf<T>::N;
+    const bool vok = (n % FV == 0) && ptj_aligned16(x) && ptj_aligned16(out) && (!dy || ptj_aligned16(dy));
+    if (n == 0) return PTJ_OK;
+    if (vok) {
+        const int64_t nvec = n / FV;
+        if (bwd)
+            hipLaunchKernelGGL((gelu_bwd_kernel<T, FV>), dim3(flat_grid(nvec)), dim3(256), 0, st, (const T*)dy,
+                               (const T*)x, (T*)out, nvec);
+        else
+            hipLaunchKernelGGL((gelu_fwd_kernel<T, FV>), dim3(flat_grid(nvec)), dim3(256), 0, st, (const T*)x, (T*)out,
+                               nvec);
+    } else {
+        if (bwd)
+            hipLaunchKernelGGL((gelu_bwd_kernel<T, 1>), dim3(flat_grid(n)), dim3(256), 0, st, (const T*)dy,
+                               (const T*)x, (T*)out, n);
+        else
+            hipLaunchKernelGGL((gelu_fwd_kernel<T, 1>), dim3(flat_grid(n)), dim3(256), 0, st, (const T*)x, (T*)out, n);
+    }
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+template <typename T>
+int dropout_impl(const void* x, const void* res, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
+                 int train, int64_t seed, hipStream_t st) {
+    constexpr int FV = VecOf<T>::N;
+    if (rows == 0 || cols == 0) return PTJ_OK;
+    const bool vok = (cols % FV == 0) && (xs % FV == 0) && (ys % FV == 0) && ptj_aligned16(x) && ptj_aligned16(y) &&
+                     (!res || ptj_aligned16(res));
+#define LAUNCH(V_, ADD_)                                                                                       \
+    hipLaunchKernelGGL((dropout_kernel<T, V_, ADD_>), dim3(flat_grid(rows * (cols / V_))), dim3(256), 0, st,     \
+                       (const T*)x, (const T*)res, (T*)y, rows, (int)cols, xs, ys, train, (uint64_t)seed)
+    if (vok) {
+        if (res) LAUNCH(FV, true); else LAUNCH(FV, false);
+    } else {
+        if (res) LAUNCH(1, true); else LAUNCH(1, false);
+    }
+#undef LAUNCH
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+#define DTYPE_SWITCH(dtype, CALL_F32, CALL_BF16)                                  \
+    switch (dtype) {                                                              \
+        case PTJ_F32: return CALL_F32;                                            \
+        case PTJ_BF16: return CALL_BF16;                                          \
+        default: return ptj_set_error(PTJ_ERR_INVALID, "%s: unknown dtype %d", __func__, dtype); \
+    }
+
+}  // namespace
+
+extern "C" {
+
+int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, int64_t rows, int64_t cols,
+                      int64_t xs, int64_t ys, int dtype, void* stream) {
+    PTJ_CHECK_ARG(x && gamma && beta && y, "layernorm_fwd: null pointer");
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 2, "layernorm_fwd: need rows >= 0 and cols >= 2 (unbiased std), got %lld x %lld",
+                  (long long)rows, (long long)cols);
+    PTJ_CHECK_ARG(xs >= cols && ys >= cols, "layernorm_fwd: row stride smaller than cols");
+    if (rows == 0) return PTJ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (layernorm_fwd_impl<float>(x, gamma, beta, y, rows, cols, xs, ys, st)),
+                 (layernorm_fwd_impl<bf16>(x, gamma, beta, y, rows, cols, xs, ys, st)));
+}
+
+size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    // Upper bound over the row configurations the dispatcher can pick.
+    int np = ln_bwd_nparts(rows, 64);
+    return (size_t)np * 2 * (size_t)cols * sizeof(float);
+}
+
+int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
+                      void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
+                      int64_t dxs, int dtype, void* stream) {
+    PTJ_CHECK_ARG(dy && x, "layernorm_bwd: null dy/x");
+    PTJ_CHECK_ARG(dx || dgamma, "layernorm_bwd: nothing to compute (dx and dgamma both null)");
+    PTJ_CHECK_ARG(!dx || gamma, "layernorm_bwd: dx requested without gamma");
+    PTJ_CHECK_ARG((dgamma == nullptr) == (dbeta == nullptr), "layernorm_bwd: dgamma and dbeta must be given together");
+    PTJ_CHECK_ARG(rows >= 1 && cols >= 2, "layernorm_bwd: need rows >= 1 and cols >= 2");
+    PTJ_CHECK_ARG(dys >= cols && xs >= cols && (!dx || dxs >= cols), "layernorm_bwd: row stride smaller than cols");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype,
+                 (layernorm_bwd_impl<float>(dy, x, gamma, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols,
+                                            dys, xs, dxs, st)),
+                 (layernorm_bwd_impl<bf16>(dy, x, gamma, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols, dys,
+                                           xs, dxs, st)));
+}
+
+int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream) {
+    PTJ_CHECK_ARG(n >= 0 && (n == 0 || (x && y)), "gelu_fwd: bad arguments");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (gelu_impl<float>(nullptr, x, y, n, false, st)), (gelu_impl<bf16>(nullptr, x, y, n, false, st)));
+}
+
+int ptj_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype, void* stream) {
+    PTJ_CHECK_ARG(n >= 0 && (n == 0 || (dy && x && dx)), "gelu_bwd: bad arguments");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (gelu_impl<float>(dy, x, dx, n, true, st)), (gelu_impl<bf16>(dy, x, dx, n, true, st)));
+}
+
+int ptj_dropout(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, int train, int64_t seed,
+                int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 0, "dropout: negative shape");
+    PTJ_CHECK_ARG(rows * cols == 0 || (x && y), "dropout: null pointer");
+    PTJ_CHECK_ARG(xs >= cols && ys >= cols, "dropout: row stride smaller than cols");
+    PTJ_CHECK_ARG(cols < (1ll << 31), "dropout: cols must fit in 31 bits");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (dropout_impl<float>(x, nullptr, y, rows, cols, xs, ys, train, seed, st)),
+                 (dropout_impl<bf16>(x, nullptr, y, rows, cols, xs, ys, train, seed, st)));
+}
+
+int ptj_dropout_add(const void* x, const void* res, void* y, int64_t rows, int64_t cols, int train, int64_t seed,
+                    int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 0, "dropout_add: negative shape");
+    PTJ_CHECK_ARG(rows * cols == 0 || (x && res && y), "dropout_add: null pointer");
+    PTJ_CHECK_ARG(cols < (1ll << 31), "dropout_add: cols must fit in 31 bits");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (dropout_impl<float>(x, res, y, rows, cols, cols, cols, train, seed, st)),
+                 (dropout_impl<bf16>(x, res, y, rows, cols, cols, cols, train, seed, st)));
+}
+
+int ptj_log_softmax_fwd(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, int dtype,
+                        void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 1, "log_softmax_fwd: bad shape");
+    PTJ_CHECK_ARG(rows == 0 || (x && y), "log_softmax_fwd: null pointer");
+    PTJ_CHECK_ARG(xs >= cols && ys >= cols, "log_softmax_fwd: row stride smaller than cols");
+    if (rows == 0) return PTJ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (log_softmax_fwd_impl<float>(x, y, rows, cols, xs, ys, st)),
+                 (log_softmax_fwd_impl<bf16>(x, y, rows, cols, xs, ys, st)));
+}
+
+int ptj_log_softmax_bwd(const void* dy, const void* x, void* dx, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
+                        int64_t dxs, int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 1, "log_softmax_bwd: bad shape");
+    PTJ_CHECK_ARG(rows == 0 || (dy && x && dx), "log_softmax_bwd: null pointer");
+    PTJ_CHECK_ARG(dys >= cols && xs >= cols && dxs >= cols, "log_softmax_bwd: row stride smaller than cols");
+    if (rows == 0) return PTJ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (log_softmax_bwd_impl<float>(dy, x, dx, rows, cols, dys, xs, dxs, st)),
+                 (log_softmax_bwd_impl<bf16>(dy, x, dx, rows, cols, dys, xs, dxs, st)));
+}
+
+}  // extern "C"

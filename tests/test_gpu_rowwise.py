@@ -1,0 +1,135 @@
+"""GPU parity of the row-wise kernels (through the C ABI) against the CPU oracle.
+Tolerances: fp32 rtol 1e-5 (+atol 1e-6); bf16 rtol 2e-2 (+atol 2e-3) against the fp64
+oracle evaluated on the bf16-rounded inputs.  Dropout masks are compared bit-exactly."""
+import pytest
+import torch
+
+from oracle import ops
+from util import DTYPES, assert_close, f64, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(8192, 768), (3, 5, 768), (7, 100), (33, 1000), (5, 4096), (2, 12000), (1, 2)])
+def test_layernorm_fwd(mt, dtype, shape):
+    g = gen(1)
+    x = randn(g, *shape, dtype=dtype)
+    D = shape[-1]
+    gamma, beta = randn(g, D, dtype=dtype, mean=1.0, std=0.1), randn(g, D, dtype=dtype, std=0.1)
+    y = mt.t_layernorm_fwd_t((gamma.to(DEV), beta.to(DEV)), x.to(DEV))
+    assert y.shape == x.shape and y.dtype == dtype
+    want = ops.layernorm_fwd((f64(gamma), f64(beta)), f64(x))
+    # D=2 rows have |xhat| = 1/sqrt(2) exactly; generic tolerance is fine
+    assert_close(y, want, dtype, what="layernorm_fwd")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(8192, 768), (4, 6, 768), (7, 100), (300, 1000), (5, 4096)])
+def test_layernorm_bwd(mt, dtype, shape):
+    g = gen(2)
+    x, dy = randn(g, *shape, dtype=dtype), randn(g, *shape, dtype=dtype)
+    D = shape[-1]
+    gamma, beta = randn(g, D, dtype=dtype, mean=1.0, std=0.1), randn(g, D, dtype=dtype, std=0.1)
+    p = (gamma.to(DEV), beta.to(DEV))
+    dx = mt.t_layernorm_bkwd2_x_t(dy.to(DEV), p, x.to(DEV))
+    dg, db = mt.t_layernorm_bkwd2_p_t(dy.to(DEV), p, x.to(DEV))
+    dx2, (dg2, db2) = mt.layernorm_bkwd2_t(dy.to(DEV), p, x.to(DEV))
+    want_dx = ops.layernorm_bkwd2_x(f64(dy), (f64(gamma),), f64(x))
+    want_dg, want_db = ops.layernorm_bkwd2_p(f64(dy), None, f64(x))
+    rows = x.numel() // D
+    # dx: cancellation of three terms of size ~|g|; atol scaled to the terms
+    assert_close(dx, want_dx, dtype, atol=2e-5 if dtype == torch.float32 else 3e-2, what="ln dx")
+    # column sums over `rows` terms of size ~1: absolute error grows like sqrt(rows)*eps
+    a = (1e-6 if dtype == torch.float32 else 8e-3) * max(1.0, rows ** 0.5)
+    assert_close(dg, want_dg, dtype, atol=a, what="ln dgamma")
+    assert_close(db, want_db, dtype, atol=a, what="ln dbeta")
+    assert torch.equal(dx, dx2) and torch.equal(dg, dg2) and torch.equal(db, db2)   # fused == separate, bitwise
+    # determinism (no atomics)
+    dg3, db3 = mt.t_layernorm_bkwd2_p_t(dy.to(DEV), p, x.to(DEV))
+    assert torch.equal(dg, dg3) and torch.equal(db, db3)
+    if dtype == torch.float32:
+        # row invariants of the unbiased-std layernorm VJP
+        xh = ops.layernorm_fwd((torch.ones(D, dtype=torch.float64), torch.zeros(D, dtype=torch.float64)), f64(x))
+        assert f64(dx).sum(-1).abs().max() < 1e-3
+        assert (f64(dx) * xh).sum(-1).abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(8192, 3072), (3, 1001), (0,), (5,)])
+def test_gelu(mt, dtype, shape):
+    g = gen(3)
+    x, dy = randn(g, *shape, dtype=dtype, std=2.0), randn(g, *shape, dtype=dtype)
+    y = mt.t_gelu_fwd_t(x.to(DEV))
+    dx = mt.t_gelu_bkwd2_t(dy.to(DEV), x.to(DEV))
+    assert y.shape == x.shape and dx.shape == x.shape
+    assert_close(y, ops.gelu(f64(x)), dtype, atol=2e-6 if dtype == torch.float32 else 2e-3, what="gelu fwd")
+    assert_close(dx, ops.gelu_bkwd2(f64(dy), f64(x)), dtype, atol=2e-6 if dtype == torch.float32 else 2e-3,
+                 what="gelu bwd")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,seed", [((8192, 768), 42), ((2, 3, 768), 7), ((5, 100), 123456), ((3, 1001), 999999),
+                                        ((4, 8), (1 << 32) + 5)])
+def test_dropout_mask_bit_exact(mt, dtype, shape, seed):
+    g = gen(4)
+    x = randn(g, *shape, dtype=dtype) + 3.0          # keep away from 0 so y != 0 <=> kept
+    y = mt.t_dropout_fwd_t(x.to(DEV), True, seed).cpu()
+    keep = ops.rowwise_keep(tuple(shape), seed)
+    assert torch.equal(y != 0, keep)                  # mask bit-exact
+    assert torch.equal(y[keep], x[keep])              # no rescale: values pass through bitwise
+    dy = randn(g, *shape, dtype=dtype) + 3.0
+    d = mt.t_dropout_bkwd2_t(dy.to(DEV), x.to(DEV), True, seed).cpu()
+    assert torch.equal(d != 0, keep) and torch.equal(d[keep], dy[keep])
+    # eval mode: x * 0.9
+    e = mt.t_dropout_fwd_t(x.to(DEV), False)
+    assert_close(e, f64(x) * 0.9, dtype, what="dropout eval")
+    # fused residual form
+    r = randn(g, *shape, dtype=dtype)
+    ya = mt.dropout_add_t(x.to(DEV), r.to(DEV), True, seed).cpu()
+    assert torch.equal(ya, (r.to(torch.float32) + y.to(torch.float32)).to(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(8, 12, 64, 512), (4096, 1024), (3, 37), (2, 4096), (5, 1)])
+def test_log_softmax(mt, dtype, shape):
+    g = gen(5)
+    x, dy = randn(g, *shape, dtype=dtype, std=3.0), randn(g, *shape, dtype=dtype)
+    y = mt.t_log_softmax_fwd_t(x.to(DEV))
+    dx = mt.t_log_softmax_bkwd2_t(dy.to(DEV), x.to(DEV))
+    a = 1e-5 if dtype == torch.float32 else 6e-2      # |y| ~ 10: bf16 spacing there is 6e-2
+    assert_close(y, ops.log_softmax(f64(x)), dtype, atol=a, what="log_softmax fwd")
+    assert_close(dx, ops.log_softmax_bkwd2(f64(dy), f64(x)), dtype, atol=1e-5 if dtype == torch.float32 else 2e-2,
+                 what="log_softmax bwd")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,V", [(512, 50257), (64, 35374), (33, 1000), (7, 101), (4, 70001), (1, 5)])
+def test_ce_fwd_bwd(lo, dtype, rows, V):
+    g = gen(6)
+    x = randn(g, rows, V, dtype=dtype)
+    y = torch.randint(0, V, (rows,), generator=g)
+    y[::7] = 0
+    if rows == 1:
+        y[0] = 3
+    loss, cnt, dx = lo.t_avg_cross_entropy_loss_bkwd3_t(y.to(DEV), x.to(DEV))
+    wl, wc, wdx = ops.avg_cross_entropy_loss_bkwd3(y, f64(x))
+    assert cnt.item() == wc.item() and cnt.dtype == torch.int64
+    assert loss.shape == (1,) and loss.dtype == torch.float32
+    assert abs(loss.item() - wl.item()) <= (1e-5 if dtype == torch.float32 else 1e-4) * abs(wl.item())
+    assert dx.shape == x.shape and dx.dtype == dtype
+    assert_close(dx, wdx, dtype, atol=1e-9 if dtype == torch.float32 else 1e-6, what="ce dlogits")
+    assert torch.equal(dx.cpu()[y == 0], torch.zeros_like(x)[y == 0])
+    # determinism + in-place variant
+    loss2, _, dx2 = lo.t_avg_cross_entropy_loss_bkwd3_t(y.to(DEV), x.to(DEV))
+    assert torch.equal(loss, loss2) and torch.equal(dx, dx2)
+    xin = x.to(DEV).clone()
+    loss3, _, dx3 = lo.t_avg_cross_entropy_loss_bkwd3_t(y.to(DEV), xin, inplace=True)
+    assert dx3.data_ptr() == xin.data_ptr() and torch.equal(dx3, dx) and torch.equal(loss3, loss)
+
+
+def test_ce_all_labels_zero_is_nan(lo):
+    x = torch.randn(4, 50, device=DEV)
+    loss, cnt, dx = lo.t_avg_cross_entropy_loss_bkwd3_t(torch.zeros(4, dtype=torch.int64, device=DEV), x)
+    assert torch.isnan(loss).all() and cnt.item() == 0 and (dx == 0).all()
