@@ -113,11 +113,17 @@ int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64
  * `.t()`), C is row-major with row stride c_rs.  Replaces t_matmul_k / t_matmul_t
  * (model_triton.py:313-398) and the two launches of t_tlayer_ffn_fwd_t (:1258-1313);
  * also the torch.matmul / einsum call sites of the training path
- * (:306, :436, :460-472, :495-508, :423-428). */
+ * (:306, :436, :460-472, :495-508, :423-428).
+ * Operands that are 16-byte aligned with a leading stride that is a multiple of
+ * 16 bytes take the vectorised path; anything else (any strides) is still computed,
+ * through scalar loads.  `workspace` (nullable) lets small outputs with a long k be
+ * split along k: pass ptj_gemm_workspace_bytes(n, m, k, dtype) bytes; the split
+ * partials are reduced in fixed order, so results are deterministic. */
+size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype);
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
              int64_t n, int64_t m, int64_t k,
              int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs,
-             int epilogue, int dtype, void* stream);
+             int epilogue, void* workspace, size_t workspace_bytes, int dtype, void* stream);
 
 /* ---- attention ----------------------------------------------------------- */
 

@@ -129,18 +129,28 @@ __device__ __forceinline__ bool philox_keep(uint32_t offset, uint32_t k0, uint32
     return x > PTJ_DROPOUT_KEEP_THRESHOLD;
 }
 
-// tanh-GELU with tanh(z) = 2*sigmoid(2z) - 1 (the reference's device formula).
-__device__ __forceinline__ float tanh_via_sigmoid(float z) {
-    return 2.0f / (1.0f + __expf(-2.0f * z)) - 1.0f;
+// tanh-GELU.  The reference evaluates tanh(z) as 2*sigmoid(2z) - 1, so that
+//   gelu(x)  = 0.5 x (1 + tanh z)                       = x * s
+//   gelu'(x) = 0.5 (1 + tanh z) + 0.5 x (1 - tanh^2 z) z' = s + 2 x s (1 - s) z'
+// with s = sigmoid(2z), z = k (x + 0.044715 x^3), z' = k (1 + 3*0.044715 x^2).
+// s and 1-s are both formed from a = exp(-2|z|) <= 1, which avoids the cancellation
+// of (1 + tanh z) for very negative z and any overflow.
+struct SigPair { float s, om; };  // s = sigmoid(2z), om = 1 - s
+__device__ __forceinline__ SigPair sigmoid2z(float z) {
+    const float a = __expf(-2.0f * fabsf(z));
+    const float r = 1.0f / (1.0f + a);
+    SigPair o;
+    o.s = z >= 0.f ? r : a * r;
+    o.om = z >= 0.f ? a * r : r;
+    return o;
 }
 __device__ __forceinline__ float gelu_f(float x) {
     constexpr float k = 0.7978845608028654f;
-    return 0.5f * x * (1.0f + tanh_via_sigmoid(k * (x + 0.044715f * x * x * x)));
+    return x * sigmoid2z(k * (x + 0.044715f * x * x * x)).s;
 }
 __device__ __forceinline__ float gelu_grad_f(float x) {
     constexpr float k = 0.7978845608028654f;
     const float x2 = x * x;
-    const float t = tanh_via_sigmoid(k * (x + 0.044715f * x * x2));
-    const float dt = (1.0f - t * t) * k * (1.0f + 3.0f * 0.044715f * x2);
-    return 0.5f * (1.0f + t) + 0.5f * x * dt;
+    const SigPair sp = sigmoid2z(k * (x + 0.044715f * x * x2));
+    return sp.s * (1.0f + 2.0f * x * sp.om * k * (1.0f + 3.0f * 0.044715f * x2));
 }

@@ -1,0 +1,403 @@
+// MFMA GEMM for gfx950: C[n,m] = sum_k A(n,k) B(k,m) (+bias[m]) (gelu), fp32 accumulation.
+//
+// Tiling: one 256-thread workgroup (4 wavefronts, 2x2) owns a 128x128 tile of C; each
+// wavefront owns 64x64 = 2x2 MFMA tiles of 32x32 (v_mfma_f32_32x32x16_bf16, or four
+// v_mfma_f32_32x32x2_f32 per step for fp32 storage).  The K dimension advances in tiles
+// of 128 BYTES per row (64 bf16 / 32 fp32), double-buffered in LDS: while the MFMAs
+// consume buffer p, the next tile travels HBM -> registers -> buffer p^1, one barrier
+// per step.
+//
+// LDS tile layout (both operands): [row][128 bytes of K], no padding, the eight 16-byte
+// chunks of a row XOR-swizzled by sw(row) = (row ^ row>>3) & 7.  A lane's MFMA operand is
+// one 16-byte chunk (8 consecutive k for bf16, 4 for fp32; lane = (row & 31, k-half)),
+// read with a single ds_read_b128 and conflict-free under the swizzle.  Operands whose
+// contiguous axis is K are copied 16 bytes at a time; operands whose contiguous axis is
+// the row/column axis (views made by .t(), needed by dX and dW products) are loaded as
+// 16-byte vectors along that axis and transposed while being written to LDS.
+//
+// The MFMA roles are swapped (MFMA-A = B tile, MFMA-B = A tile) so that each lane ends
+// up with 4 consecutive columns of one C row; the tile is staged through LDS in fp32 and
+// written back with full-row coalesced stores after the bias/GELU epilogue.
+//
+// Workgroup -> tile mapping: ids are first regrouped so that the workgroups that land on
+// one XCD (id mod 8) cover a contiguous range of tiles (they share that XCD's L2), then
+// walked in groups of 8 tile-rows.  Small outputs with a long K (the dW products) are
+// split along K across gridDim.z into an fp32 workspace and reduced in fixed order.
+#include "common.h"
+
+namespace {
+
+constexpr int BM = 128, BN = 128;       // C tile (rows from A, columns from B)
+constexpr int BKB = 128;                // bytes of K per tile row
+constexpr int GEMM_THREADS = 256;
+constexpr int STAGE_PITCH = 64 * 4 + 16;  // bytes per staged fp32 row of a 64x64 wave tile
+
+enum LoadMode { KMAJOR = 0, MNMAJOR = 1, GENERIC = 2 };
+
+__device__ __forceinline__ int sw(int row) { return (row ^ (row >> 3)) & 7; }
+
+template <typename T> struct Frag;
+template <> struct Frag<bf16> { typedef bf16x8 type; };
+template <> struct Frag<float> { typedef f32x4 type; };
+
+__device__ __forceinline__ void mma_chunk(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_chunk(f32x16& acc, const f32x4& a, const f32x4& b) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], acc, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------
+// Operand tile loader: 128 rows x (BKB/sizeof(T)) k-values, HBM -> registers -> LDS.
+// `row` is the C-row (operand A) or C-column (operand B) index, `k` the contraction index.
+//   KMAJOR : element(row,k) = p[row*ld + k]
+//   MNMAJOR: element(row,k) = p[k*ld + row]
+//   GENERIC: element(row,k) = p[row*s_row + k*s_k], scalar loads, any strides/alignment
+// ---------------------------------------------------------------------------------
+template <typename T, int MODE>
+struct TileLoader {
+    static constexpr int VEC = VecOf<T>::N;
+    static constexpr int BK = BKB / (int)sizeof(T);
+    Pack<T, VEC> r[4];
+
+    __device__ __forceinline__ void load(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int nrows,
+                                         int k0, int kend, int tid) {
+        if constexpr (MODE == KMAJOR || MODE == GENERIC) {
+            const int c = tid & 7;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = row0 + (tid >> 3) + 32 * i;
+                const int k = k0 + c * VEC;
+                if (MODE == KMAJOR && row < nrows && k + VEC <= kend) {
+                    r[i] = *reinterpret_cast<const Pack<T, VEC>*>(p + (int64_t)row * s_row + k);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        r[i].v[e] = (row < nrows && k + e < kend) ? p[(int64_t)row * s_row + (int64_t)(k + e) * s_k]
+                                                                  : from_f32<T>(0.f);
+                }
+            }
+        } else {
+            // block b = wave*4 + i covers 8 row-vectors x 8 k; blocks tile (128/VEC/8) x (BK/8)
+            constexpr int JG = BM / VEC / 8;
+            const int jc_lo = tid & 7, kk = (tid >> 3) & 7, w = tid >> 6;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int b = w * 4 + i;
+                const int jc = (b % JG) * 8 + jc_lo;
+                const int k = k0 + (b / JG) * 8 + kk;
+                const int row = row0 + jc * VEC;
+                if (k < kend && row + VEC <= nrows) {
+                    r[i] = *reinterpret_cast<const Pack<T, VEC>*>(p + (int64_t)k * s_k + row);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        r[i].v[e] = (k < kend && row + e < nrows) ? p[(int64_t)k * s_k + row + e] : from_f32<T>(0.f);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(char* __restrict__ lds, int tid) const {
+        if constexpr (MODE == KMAJOR || MODE == GENERIC) {
+            const int c = tid & 7;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = (tid >> 3) + 32 * i;
+                *reinterpret_cast<Pack<T, VEC>*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
+            }
+        } else {
+            constexpr int JG = BM / VEC / 8;
+            const int jc_lo = tid & 7, kk = (tid >> 3) & 7, w = tid >> 6;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int b = w * 4 + i;
+                const int jc = (b % JG) * 8 + jc_lo;
+                const int kb = ((b / JG) * 8 + kk) * (int)sizeof(T);  // byte offset of k inside the row
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const int row = jc * VEC + e;
+                    *reinterpret_cast<T*>(lds + row * BKB + (((kb >> 4) ^ sw(row)) << 4) + (kb & 15)) = r[i].v[e];
+                }
+            }
+        }
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ typename Frag<T>::type read_frag(const char* __restrict__ lds, int row, int q) {
+    return *reinterpret_cast<const typename Frag<T>::type*>(lds + row * BKB + ((q ^ sw(row)) << 4));
+}
+
+struct GemmArgs {
+    const void* a;
+    const void* b;
+    void* c;
+    const void* bias;
+    float* partial;   // split-K workspace [splits][n][m] (nullptr when splits == 1)
+    int n, m, k;
+    int64_t a_row, a_k;   // strides of A(row=n, k)
+    int64_t b_row, b_k;   // strides of B(row=m, k)  (b_row = b_cs, b_k = b_rs)
+    int64_t c_rs;
+    int k_per_split;      // multiple of BK
+    int epilogue;
+};
+
+template <typename T, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_kernel(const GemmArgs g) {
+    constexpr int BK = BKB / (int)sizeof(T);
+    // 64 KiB of operand tiles; the epilogue reuses it for 4 staged wave tiles (68 KiB)
+    constexpr int SMEM_BYTES = 4 * 64 * STAGE_PITCH > 2 * (BM + BN) * BKB ? 4 * 64 * STAGE_PITCH : 2 * (BM + BN) * BKB;
+    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
+    auto sA = [&](int p) -> char* { return smem + p * (BM * BKB); };
+    auto sB = [&](int p) -> char* { return smem + 2 * BM * BKB + p * (BN * BKB); };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;     // wave position in the 2x2 grid
+    const int lr = lane & 31, lg = lane >> 5;
+
+    // ---- workgroup -> tile ---------------------------------------------------------
+    const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
+    const int total = num_m * num_n;
+    int pid = blockIdx.x;
+    {
+        const int chunk = total >> 3, rem = total & 7, x = pid & 7;
+        pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
+    }
+    constexpr int GROUP = 8;
+    const int width = GROUP * num_n;
+    const int group_id = pid / width;
+    const int first_m = group_id * GROUP;
+    const int gsz = (num_m - first_m) < GROUP ? (num_m - first_m) : GROUP;
+    const int tile_m = first_m + (pid % width) % gsz;
+    const int tile_n = (pid % width) / gsz;
+    const int row0 = tile_m * BM, col0 = tile_n * BN;
+
+    const int kbeg = blockIdx.z * g.k_per_split;
+    const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
+    const int nk = (kend - kbeg + BK - 1) / BK;
+
+    const T* A = (const T*)g.a;
+    const T* B = (const T*)g.b;
+
+    f32x16 acc[2][2];  // [tn][tm]
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    TileLoader<T, AMODE> la;
+    TileLoader<T, BMODE> lb;
+    if (nk > 0) {
+        la.load(A, g.a_row, g.a_k, row0, g.n, kbeg, kend, tid);
+        lb.load(B, g.b_row, g.b_k, col0, g.m, kbeg, kend, tid);
+        la.store(sA(0), tid);
+        lb.store(sB(0), tid);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int p = kt & 1;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            la.load(A, g.a_row, g.a_k, row0, g.n, kbeg + (kt + 1) * BK, kend, tid);
+            lb.load(B, g.b_row, g.b_k, col0, g.m, kbeg + (kt + 1) * BK, kend, tid);
+        }
+        const char* cA = sA(p);
+        const char* cB = sB(p);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int q = c * 2 + lg;
+            typename Frag<T>::type fa[2], fb[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                fa[t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q);  // C rows   -> MFMA B operand
+                fb[t] = read_frag<T>(cB, wn * 64 + t * 32 + lr, q);  // C columns-> MFMA A operand
+            }
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < 2; ++tm) mma_chunk(acc[tn][tm], fb[tn], fa[tm]);
+        }
+        if (more) {
+            la.store(sA(p ^ 1), tid);
+            lb.store(sB(p ^ 1), tid);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: stage the wave's 64x64 fp32 tile in LDS, then coalesced row stores --
+    // acc[tn][tm][i] of lane (lr, lg) = C[wm*64 + tm*32 + lr][wn*64 + tn*32 + (i/4)*8 + lg*4 + (i%4)]
+    char* stage = smem + wave * (64 * STAGE_PITCH);
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                f32x4 v = {acc[tn][tm][i4 * 4 + 0], acc[tn][tm][i4 * 4 + 1], acc[tn][tm][i4 * 4 + 2],
+                           acc[tn][tm][i4 * 4 + 3]};
+                const int r = tm * 32 + lr, cc = tn * 32 + i4 * 8 + lg * 4;
+                *reinterpret_cast<f32x4*>(stage + r * STAGE_PITCH + cc * 4) = v;
+            }
+    __syncthreads();
+
+    const int cc4 = (lane & 15) * 4;          // 4 consecutive columns
+    const int gcol = col0 + wn * 64 + cc4;
+    float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (g.epilogue != PTJ_EPI_NONE && g.partial == nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (gcol + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol + e]);
+    }
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+        const int r = (lane >> 4) + 4 * it;
+        const int grow = row0 + wm * 64 + r;
+        f32x4 v = *reinterpret_cast<const f32x4*>(stage + r * STAGE_PITCH + cc4 * 4);
+        if (grow >= g.n || gcol >= g.m) continue;
+        if (g.partial != nullptr) {
+            float* dst = g.partial + ((int64_t)blockIdx.z * g.n + grow) * g.m + gcol;
+            if (gcol + 4 <= g.m && (((uintptr_t)dst & 15) == 0)) {
+                *reinterpret_cast<f32x4*>(dst) = v;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (gcol + e < g.m) dst[e] = v[e];
+            }
+            continue;
+        }
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = v[e] + bias4[e];
+            if (g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
+        }
+        T* dst = (T*)g.c + (int64_t)grow * g.c_rs + gcol;
+        if (gcol + 4 <= g.m && (((uintptr_t)dst & (4 * sizeof(T) - 1)) == 0)) {
+            store_vec<T, 4>(dst, o);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (gcol + e < g.m) dst[e] = from_f32<T>(o[e]);
+        }
+    }
+}
+
+// Split-K second stage: C = epilogue(sum_z partial[z]) in z order.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial, int splits, int n,
+                                                                  int m, T* __restrict__ c, int64_t c_rs,
+                                                                  const T* __restrict__ bias, int epilogue) {
+    const int64_t total = (int64_t)n * m;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        float s = 0.f;
+        for (int z = 0; z < splits; ++z) s += partial[z * total + i];
+        const int row = (int)(i / m), col = (int)(i - (int64_t)row * m);
+        if (epilogue != PTJ_EPI_NONE) s += to_f32(bias[col]);
+        if (epilogue == PTJ_EPI_BIAS_GELU) s = gelu_f(s);
+        c[(int64_t)row * c_rs + col] = from_f32<T>(s);
+    }
+}
+
+template <typename T>
+int pick_mode(const void* p, int64_t s_row, int64_t s_k) {
+    constexpr int VEC = VecOf<T>::N;
+    if (!ptj_aligned16(p)) return GENERIC;
+    if (s_k == 1 && s_row % VEC == 0) return KMAJOR;
+    if (s_row == 1 && s_k % VEC == 0) return MNMAJOR;
+    return GENERIC;
+}
+
+template <typename T>
+int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
+    const int am = pick_mode<T>(g.a, g.a_row, g.a_k), bm = pick_mode<T>(g.b, g.b_row, g.b_k);
+    const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
+    dim3 grid(num_m * num_n, 1, splits), block(GEMM_THREADS);
+#define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD>), grid, block, 0, st, g)
+    switch (am * 3 + bm) {
+        case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
+        case 1: GEMM_LAUNCH(KMAJOR, MNMAJOR); break;
+        case 2: GEMM_LAUNCH(KMAJOR, GENERIC); break;
+        case 3: GEMM_LAUNCH(MNMAJOR, KMAJOR); break;
+        case 4: GEMM_LAUNCH(MNMAJOR, MNMAJOR); break;
+        case 5: GEMM_LAUNCH(MNMAJOR, GENERIC); break;
+        case 6: GEMM_LAUNCH(GENERIC, KMAJOR); break;
+        case 7: GEMM_LAUNCH(GENERIC, MNMAJOR); break;
+        default: GEMM_LAUNCH(GENERIC, GENERIC); break;
+    }
+#undef GEMM_LAUNCH
+    PTJ_CHECK_LAUNCH();
+    if (splits > 1) {
+        const int64_t total = (int64_t)g.n * g.m;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 256 * 8) blocks = 256 * 8;
+        hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st,
+                           (const float*)g.partial, splits, g.n, g.m, (T*)g.c, g.c_rs, (const T*)g.bias, g.epilogue);
+        PTJ_CHECK_LAUNCH();
+    }
+    return PTJ_OK;
+}
+
+// Number of K splits for an (n, m, k) problem given `ws_bytes` of workspace.
+int choose_splits(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes) {
+    const int64_t tiles = ((n + BM - 1) / BM) * ((m + BN - 1) / BN);
+    const int bk = BKB / elt;
+    if (tiles >= 256 || k < 16 * bk) return 1;
+    int64_t s = (512 + tiles - 1) / tiles;          // aim at ~2 workgroups per CU
+    const int64_t max_by_k = k / (8 * bk);          // at least 8 K-steps per split
+    if (s > max_by_k) s = max_by_k;
+    if (s > 32) s = 32;
+    while (s > 1 && (size_t)s * n * m * sizeof(float) > ws_bytes) --s;
+    return s < 1 ? 1 : (int)s;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype) {
+    if (n <= 0 || m <= 0 || k <= 0) return 0;
+    const int elt = dtype == PTJ_BF16 ? 2 : 4;
+    const int s = choose_splits(n, m, k, elt, (size_t)-1);
+    return s > 1 ? (size_t)s * n * m * sizeof(float) : 0;
+}
+
+int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n, int64_t m, int64_t k, int64_t a_rs,
+             int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs, int epilogue, void* workspace,
+             size_t workspace_bytes, int dtype, void* stream) {
+    PTJ_CHECK_ARG(n >= 0 && m >= 0 && k >= 0, "gemm: negative dimension");
+    PTJ_CHECK_ARG(n < (1ll << 31) && m < (1ll << 31) && k < (1ll << 31), "gemm: dimension exceeds 31 bits");
+    PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_BIAS_GELU, "gemm: unknown epilogue %d", epilogue);
+    PTJ_CHECK_ARG(epilogue == PTJ_EPI_NONE || bias, "gemm: epilogue %d needs a bias", epilogue);
+    PTJ_CHECK_ARG(dtype == PTJ_F32 || dtype == PTJ_BF16, "gemm: unknown dtype %d", dtype);
+    if (n == 0 || m == 0) return PTJ_OK;
+    PTJ_CHECK_ARG(c && (k == 0 || (a && b)), "gemm: null pointer");
+    PTJ_CHECK_ARG(c_rs >= m, "gemm: c row stride %lld < m %lld", (long long)c_rs, (long long)m);
+    const int elt = dtype == PTJ_BF16 ? 2 : 4;
+    const int bk = BKB / elt;
+    GemmArgs g;
+    g.a = a; g.b = b; g.c = c; g.bias = bias;
+    g.n = (int)n; g.m = (int)m; g.k = (int)k;
+    g.a_row = a_rs; g.a_k = a_cs;
+    g.b_row = b_cs; g.b_k = b_rs;
+    g.c_rs = c_rs;
+    g.epilogue = epilogue;
+    int splits = workspace ? choose_splits(n, m, k, elt, workspace_bytes) : 1;
+    int64_t kps = k;
+    if (splits > 1) {
+        kps = ((k + splits - 1) / splits + bk - 1) / bk * bk;
+        splits = (int)((k + kps - 1) / kps);
+    }
+    if (kps < 1) kps = bk;  // k == 0: one empty pass writes bias / zeros
+    g.k_per_split = (int)kps;
+    g.partial = splits > 1 ? (float*)workspace : nullptr;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
+}
+
+}  // extern "C"

@@ -92,12 +92,18 @@ __global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_fwd_kernel(
 // Partials layout: part[p][0][cols] = sum dy*xhat, part[p][1][cols] = sum dy over the
 // rows handled by row-slot p (p = blockIdx.x*RPB + sub).
 // ---------------------------------------------------------------------------------
+template <int TPR> struct LnBwdGeom {
+    static constexpr int BLOCK = TPR == 64 ? 512 : TPR;
+    static constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
+};
+constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave holds (bf16, ITERS 4)
+
 template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
-__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
+__global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, T* __restrict__ dx,
     float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs) {
     __shared__ float smem[16];
-    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    constexpr int RPB = LnBwdGeom<TPR>::ROWS_PER_BLOCK;
     const int t = threadIdx.x % TPR;
     const int sub = threadIdx.x / TPR;
     const int nvec = cols / VEC;
@@ -167,17 +173,43 @@ __global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
         }
     }
     if constexpr (DGB) {
-        const int64_t p = (int64_t)blockIdx.x * RPB + sub;
-        float* pg = part + p * 2 * (int64_t)cols;
+        // One partial per workgroup.  With several row slots per workgroup the slots are
+        // folded through LDS in slot order (deterministic).
+        float* pg = part + (int64_t)blockIdx.x * 2 * (int64_t)cols;
         float* pb = pg + cols;
+        if constexpr (RPB > 1) {
+            __shared__ float red[2][LN_BWD_MAX_WAVE_COLS];
+            for (int s = 0; s < RPB; ++s) {
+                if (sub == s) {
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int vi = t + it * TPR;
-            if (vi < nvec) {
+                    for (int it = 0; it < ITERS; ++it) {
+                        const int vi = t + it * TPR;
+                        if (vi < nvec) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    pg[vi * VEC + j] = acc_g[it][j];
-                    pb[vi * VEC + j] = acc_b[it][j];
+                            for (int j = 0; j < VEC; ++j) {
+                                const int c = vi * VEC + j;
+                                red[0][c] = s == 0 ? acc_g[it][j] : red[0][c] + acc_g[it][j];
+                                red[1][c] = s == 0 ? acc_b[it][j] : red[1][c] + acc_b[it][j];
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+            for (int c = threadIdx.x; c < cols; c += LnBwdGeom<TPR>::BLOCK) {
+                pg[c] = red[0][c];
+                pb[c] = red[1][c];
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int vi = t + it * TPR;
+                if (vi < nvec) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        pg[vi * VEC + j] = acc_g[it][j];
+                        pb[vi * VEC + j] = acc_b[it][j];
+                    }
                 }
             }
         }
@@ -415,7 +447,13 @@ int layernorm_fwd_impl(const void* x, const void* gamma, const void* beta, void*
     return PTJ_OK;
 }
 
-inline int ln_bwd_nparts(int64_t rows, int tpr) { return row_grid(rows, tpr) * (tpr == 64 ? 4 : 1); }
+// Grid of the backward kernel = number of dgamma/dbeta partials (one per workgroup).
+inline int ln_bwd_grid(int64_t rows, int tpr) {
+    const int rpb = tpr == 64 ? 8 : 1;
+    const int64_t need = (rows + rpb - 1) / rpb;
+    const int64_t cap = 512;  // 2 workgroups per CU: bounds the partials to 512 rows of 2*cols floats
+    return (int)(need < cap ? need : cap);
+}
 
 template <typename T>
 int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
@@ -425,8 +463,8 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* d
     const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx}, {dys, xs, dx ? dxs : 0});
     if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
         return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: cols=%lld too large", (long long)cols);
-    const int grid = row_grid(rows, cfg.tpr);
-    const int nparts = ln_bwd_nparts(rows, cfg.tpr);
+    const int grid = ln_bwd_grid(rows, cfg.tpr);
+    const int nparts = grid;
     const bool want_dx = dx != nullptr, want_dgb = dgamma != nullptr;
     if (want_dgb) {
         const size_t need = (size_t)nparts * 2 * (size_t)cols * sizeof(float);
@@ -435,7 +473,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* d
     }
 #define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_)                                                                   \
     hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
-                       dim3(RowGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (T_*)dx, \
+                       dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (T_*)dx, \
                        (float*)ws, rows, (int)cols, dys, xs, dxs)
 #define LAUNCH(T_, V_, TPR_, IT_)                                     \
     do {                                                              \
@@ -566,8 +604,7 @@ int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* 
 size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     // Upper bound over the row configurations the dispatcher can pick.
-    int np = ln_bwd_nparts(rows, 64);
-    return (size_t)np * 2 * (size_t)cols * sizeof(float);
+    return (size_t)512 * 2 * (size_t)cols * sizeof(float);
 }
 
 int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,

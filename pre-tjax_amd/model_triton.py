@@ -172,3 +172,62 @@ def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor):
     launches at model_triton.py:2033-2034)."""
     dx, dg, db = _layernorm_bwd(dloss_dx, layer_params, x, True, True)
     return dx, (dg, db)
+
+
+# ----------------------------------------------------------------------------------
+# GEMM  (reference: model_triton.py:373-398 t_matmul_t, :1258-1313 t_tlayer_ffn_fwd_t)
+# ----------------------------------------------------------------------------------
+def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None):
+    """``out[N,M] = a[N,K] @ b[K,M] (+ bias[M]) (tanh-GELU)`` on the MFMA GEMM kernel.
+
+    `a` and `b` are 2-D tensors with arbitrary strides (``.t()`` views are consumed in
+    place, never copied); `out`, if given, is a 2-D tensor with unit column stride
+    (a column slice of a wider buffer is fine)."""
+    require_gpu(a, b, bias, out)
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], (a.shape, b.shape)
+    assert a.dtype == b.dtype
+    N, K = a.shape
+    M = b.shape[1]
+    if out is None:
+        out = torch.empty((N, M), dtype=a.dtype, device=a.device)
+    else:
+        assert out.shape == (N, M) and out.dtype == a.dtype and (out.stride(1) == 1 or M == 1)
+    epi = _lib.EPI_NONE
+    if bias is not None:
+        assert bias.dtype == a.dtype and bias.numel() == M
+        bias = bias.contiguous()
+        epi = _lib.EPI_BIAS_GELU if gelu else _lib.EPI_BIAS
+    else:
+        assert not gelu, "GELU epilogue is defined on top of the bias epilogue"
+    code = dtype_code(a)
+    ws_bytes = lib().ptj_gemm_workspace_bytes(N, M, K, code)
+    ws = _workspace(ws_bytes, a.device, "gemm") if ws_bytes else None
+    check(lib().ptj_gemm(ptr(a), ptr(b), ptr(out), ptr(bias), N, M, K, a.stride(0), a.stride(1), b.stride(0),
+                         b.stride(1), out.stride(0), epi, ptr(ws), ws_bytes, code, stream()), "ptj_gemm")
+    return out
+
+
+def t_matmul_t(a: torch.Tensor, b: torch.Tensor):
+    """Reference signature (model_triton.py:373): a[N,K] contiguous, b[K,M] any strides."""
+    assert a.is_contiguous(), "Matrix A must be contiguous"
+    return matmul_t(a, b)
+
+
+t_matmul = t_matmul_t
+
+
+def t_gelu_fwd(x):
+    """Marker for `activation_fn` arguments (the reference passes its torch GELU here,
+    model_triton.py:221); evaluating it runs the HIP kernel."""
+    return t_gelu_fwd_t(x)
+
+
+def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
+    """Two GEMM launches: bias+GELU epilogue, then bias (model_triton.py:1258-1313)."""
+    assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU epilogue exists"
+    w1, b1, w2, b2 = layer_params
+    shape = x.shape
+    x2 = _rows2d(x)
+    mid = matmul_t(x2, w1.t(), b1, gelu=True)
+    out = matmul_t(mid, w2.t(), b2)
+    return out.view(shape[:-1] + (w2.shape[0],))

@@ -1,0 +1,99 @@
+"""GPU parity of the MFMA GEMM (through the C ABI) against fp64 matmul of the same inputs.
+Error bound per element: tol * sum_k |a_ik b_kj| (the standard forward bound), tol = 1e-5 for
+fp32 storage and 2e-2 for bf16 storage (output rounding 2^-9 relative + accumulation)."""
+import pytest
+import torch
+
+from oracle import ops
+from util import DTYPES, f64, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def check(c, a, b, dtype, bias=None, gelu=False):
+    a64, b64 = f64(a), f64(b)
+    want = a64 @ b64
+    scale = a64.abs() @ b64.abs()
+    if bias is not None:
+        want = want + f64(bias)
+        scale = scale + f64(bias).abs()
+    if gelu:
+        want = ops.gelu(want)        # |gelu'| <= 1.13, same bound up to that factor
+        scale = scale * 1.2
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    err = (f64(c) - want).abs()
+    bound = tol * scale + (1e-30 if dtype == torch.float32 else 4e-3 * want.abs() + 1e-6)
+    assert c.shape == want.shape
+    bad = err > bound
+    assert not bad.any(), "max err/bound %.3f at %d elements" % ((err / bound).max().item(), int(bad.sum()))
+
+
+SHAPES = [(128, 128, 64), (256, 384, 512), (100, 37, 19), (513, 129, 65), (1, 1, 1), (64, 768, 3072),
+          (33, 2, 200), (300, 50257, 64)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,m,k", SHAPES)
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_gemm_layouts(mt, dtype, n, m, k, layout):
+    g = gen(n * 7 + m * 3 + k)
+    a = randn(g, n, k, dtype=dtype) if layout[0] == "n" else randn(g, k, n, dtype=dtype).t()
+    b = randn(g, k, m, dtype=dtype) if layout[1] == "n" else randn(g, m, k, dtype=dtype).t()
+    ad = (a.t().contiguous().to(DEV).t() if layout[0] == "t" else a.to(DEV))
+    bd = (b.t().contiguous().to(DEV).t() if layout[1] == "t" else b.to(DEV))
+    assert ad.stride() == a.stride() and bd.stride() == b.stride()
+    c = mt.matmul_t(ad, bd)
+    check(c, a, b, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_bruteforce_tiny(mt, dtype):
+    g = gen(5)
+    a, b = randn(g, 9, 13, dtype=dtype), randn(g, 13, 6, dtype=dtype)
+    c = mt.t_matmul_t(a.to(DEV), b.to(DEV))
+    want = ops.matmul_bruteforce(f64(a), f64(b))
+    assert torch.allclose(f64(c), want, rtol=1e-5 if dtype == torch.float32 else 2e-2, atol=1e-5 if dtype == torch.float32 else 5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,m,k", [(768, 768, 16384), (2304, 768, 8192), (50257, 64, 4096), (130, 70, 5000)])
+def test_gemm_split_k_dw_shapes(mt, dtype, n, m, k):
+    # dW-like products: both operands contiguous along the output axes, long contraction
+    g = gen(11)
+    dy, x = randn(g, k, n, dtype=dtype), randn(g, k, m, dtype=dtype)
+    c = mt.matmul_t(dy.to(DEV).t(), x.to(DEV))
+    check(c, dy.t(), x, dtype)
+    c2 = mt.matmul_t(dy.to(DEV).t(), x.to(DEV))
+    assert torch.equal(c, c2)      # split-K partials are reduced in fixed order
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_bias_gelu_and_ffn(mt, dtype):
+    g = gen(12)
+    x = randn(g, 4, 96, 768, dtype=dtype)
+    w1, b1 = randn(g, 3072, 768, dtype=dtype, std=0.02), randn(g, 3072, dtype=dtype, std=0.1)
+    w2, b2 = randn(g, 768, 3072, dtype=dtype, std=0.02), randn(g, 768, dtype=dtype, std=0.1)
+    x2 = x.reshape(-1, 768)
+    h = mt.matmul_t(x2.to(DEV), w1.to(DEV).t(), b1.to(DEV), gelu=True)
+    check(h, x2, w1.t(), dtype, bias=b1, gelu=True)
+    y = mt.t_tlayer_ffn_fwd_t((w1.to(DEV), b1.to(DEV), w2.to(DEV), b2.to(DEV)), x.to(DEV), mt.t_gelu_fwd)
+    assert y.shape == x.shape
+    want = ops.gelu(f64(x2) @ f64(w1).t() + f64(b1)) @ f64(w2).t() + f64(b2)
+    rel = ((f64(y).reshape(-1, 768) - want).norm() / want.norm()).item()
+    assert rel < (1e-5 if dtype == torch.float32 else 1e-2), rel
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_strided_output_and_misaligned_inputs(mt, dtype):
+    g = gen(13)
+    a, b = randn(g, 70, 41, dtype=dtype), randn(g, 41, 50, dtype=dtype)
+    buf = torch.zeros(70, 64, dtype=dtype, device=DEV)
+    mt.matmul_t(a.to(DEV), b.to(DEV), out=buf[:, :50])
+    check(buf[:, :50], a, b, dtype)
+    assert (buf[:, 50:] == 0).all()
+    # operands starting 1 element into an allocation (not 16-byte aligned)
+    pa = torch.zeros(70 * 41 + 1, dtype=dtype, device=DEV)
+    pa[1:] = a.to(DEV).reshape(-1)
+    c = mt.matmul_t(pa[1:].view(70, 41), b.to(DEV))
+    check(c, a, b, dtype)

@@ -42,7 +42,7 @@ def test_layernorm_bwd(mt, dtype, shape):
     # dx: cancellation of three terms of size ~|g|; atol scaled to the terms
     assert_close(dx, want_dx, dtype, atol=2e-5 if dtype == torch.float32 else 3e-2, what="ln dx")
     # column sums over `rows` terms of size ~1: absolute error grows like sqrt(rows)*eps
-    a = (1e-6 if dtype == torch.float32 else 8e-3) * max(1.0, rows ** 0.5)
+    a = (3e-6 if dtype == torch.float32 else 8e-3) * max(1.0, rows ** 0.5)
     assert_close(dg, want_dg, dtype, atol=a, what="ln dgamma")
     assert_close(db, want_db, dtype, atol=a, what="ln dbeta")
     assert torch.equal(dx, dx2) and torch.equal(dg, dg2) and torch.equal(db, db2)   # fused == separate, bitwise
@@ -74,12 +74,12 @@ def test_gelu(mt, dtype, shape):
                                         ((4, 8), (1 << 32) + 5)])
 def test_dropout_mask_bit_exact(mt, dtype, shape, seed):
     g = gen(4)
-    x = randn(g, *shape, dtype=dtype) + 3.0          # keep away from 0 so y != 0 <=> kept
+    x = randn(g, *shape, dtype=dtype).abs() + 1.0    # strictly positive so y != 0 <=> kept
     y = mt.t_dropout_fwd_t(x.to(DEV), True, seed).cpu()
     keep = ops.rowwise_keep(tuple(shape), seed)
     assert torch.equal(y != 0, keep)                  # mask bit-exact
     assert torch.equal(y[keep], x[keep])              # no rescale: values pass through bitwise
-    dy = randn(g, *shape, dtype=dtype) + 3.0
+    dy = randn(g, *shape, dtype=dtype).abs() + 1.0
     d = mt.t_dropout_bkwd2_t(dy.to(DEV), x.to(DEV), True, seed).cpu()
     assert torch.equal(d != 0, keep) and torch.equal(d[keep], dy[keep])
     # eval mode: x * 0.9
