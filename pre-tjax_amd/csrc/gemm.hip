@@ -1,134 +1,38 @@
 // MFMA GEMM for gfx950: C[n,m] = sum_k A(n,k) B(k,m) (+bias[m]) (gelu), fp32 accumulation.
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2x2) owns a 128x128 tile of C; each
-// wavefront owns 64x64 = 2x2 MFMA tiles of 32x32 (v_mfma_f32_32x32x16_bf16, or four
-// v_mfma_f32_32x32x2_f32 per step for fp32 storage).  The K dimension advances in tiles
-// of 128 BYTES per row (64 bf16 / 32 fp32), double-buffered in LDS: while the MFMAs
-// consume buffer p, the next tile travels HBM -> registers -> buffer p^1, one barrier
-// per step.
+// Tiling: one 512-thread workgroup (8 wavefronts, 4 along rows x 2 along columns) owns a
+// 256x192 tile of C; each wavefront owns 64x96 = 2x3 MFMA tiles of 32x32
+// (v_mfma_f32_32x32x16_bf16, or four v_mfma_f32_32x32x2_f32 per step for fp32 storage).
+// 192 divides every feature width of the model (768, 2304, 3072) and 256 divides B*T, so
+// the big products fill the 256 CUs in whole rounds.  K advances in panels of 128 BYTES
+// per row (64 bf16 / 32 fp32), double-buffered in LDS (2 x 56 KiB): while the MFMAs
+// consume buffer p, the next panels travel HBM -> registers -> buffer p^1, one barrier
+// per step; two wavefronts per SIMD overlap one's MFMAs with the other's copies.
 //
-// LDS tile layout (both operands): [row][128 bytes of K], no padding, the eight 16-byte
-// chunks of a row XOR-swizzled by sw(row) = (row ^ row>>3) & 7.  A lane's MFMA operand is
-// one 16-byte chunk (8 consecutive k for bf16, 4 for fp32; lane = (row & 31, k-half)),
-// read with a single ds_read_b128 and conflict-free under the swizzle.  Operands whose
-// contiguous axis is K are copied 16 bytes at a time; operands whose contiguous axis is
-// the row/column axis (views made by .t(), needed by dX and dW products) are loaded as
-// 16-byte vectors along that axis and transposed while being written to LDS.
+// LDS panels and their swizzle are described in mma_tile.h.  Operands whose contiguous
+// axis is K are copied 16 bytes at a time; operands whose contiguous axis is the
+// row/column axis (.t() views: the dX and dW products) are transposed in registers on
+// the way in.
 //
-// The MFMA roles are swapped (MFMA-A = B tile, MFMA-B = A tile) so that each lane ends
+// The MFMA roles are swapped (MFMA-A = B panel, MFMA-B = A panel) so that each lane ends
 // up with 4 consecutive columns of one C row; the tile is staged through LDS in fp32 and
-// written back with full-row coalesced stores after the bias/GELU epilogue.
+// written back with row-contiguous stores after the bias/GELU epilogue.
 //
 // Workgroup -> tile mapping: ids are first regrouped so that the workgroups that land on
 // one XCD (id mod 8) cover a contiguous range of tiles (they share that XCD's L2), then
 // walked in groups of 8 tile-rows.  Small outputs with a long K (the dW products) are
 // split along K across gridDim.z into an fp32 workspace and reduced in fixed order.
 #include "common.h"
+#include "mma_tile.h"
+#include <type_traits>
 
 namespace {
 
-constexpr int BM = 128, BN = 128;       // C tile (rows from A, columns from B)
-constexpr int BKB = 128;                // bytes of K per tile row
-constexpr int GEMM_THREADS = 256;
-constexpr int STAGE_PITCH = 64 * 4 + 16;  // bytes per staged fp32 row of a 64x64 wave tile
-
-enum LoadMode { KMAJOR = 0, MNMAJOR = 1, GENERIC = 2 };
-
-__device__ __forceinline__ int sw(int row) { return (row ^ (row >> 3)) & 7; }
-
-template <typename T> struct Frag;
-template <> struct Frag<bf16> { typedef bf16x8 type; };
-template <> struct Frag<float> { typedef f32x4 type; };
-
-__device__ __forceinline__ void mma_chunk(f32x16& acc, const bf16x8& a, const bf16x8& b) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
-}
-__device__ __forceinline__ void mma_chunk(f32x16& acc, const f32x4& a, const f32x4& b) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], acc, 0, 0, 0);
-}
-
-// ---------------------------------------------------------------------------------
-// Operand tile loader: 128 rows x (BKB/sizeof(T)) k-values, HBM -> registers -> LDS.
-// `row` is the C-row (operand A) or C-column (operand B) index, `k` the contraction index.
-//   KMAJOR : element(row,k) = p[row*ld + k]
-//   MNMAJOR: element(row,k) = p[k*ld + row]
-//   GENERIC: element(row,k) = p[row*s_row + k*s_k], scalar loads, any strides/alignment
-// ---------------------------------------------------------------------------------
-template <typename T, int MODE>
-struct TileLoader {
-    static constexpr int VEC = VecOf<T>::N;
-    static constexpr int BK = BKB / (int)sizeof(T);
-    Pack<T, VEC> r[4];
-
-    __device__ __forceinline__ void load(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int nrows,
-                                         int k0, int kend, int tid) {
-        if constexpr (MODE == KMAJOR || MODE == GENERIC) {
-            const int c = tid & 7;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = row0 + (tid >> 3) + 32 * i;
-                const int k = k0 + c * VEC;
-                if (MODE == KMAJOR && row < nrows && k + VEC <= kend) {
-                    r[i] = *reinterpret_cast<const Pack<T, VEC>*>(p + (int64_t)row * s_row + k);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e)
-                        r[i].v[e] = (row < nrows && k + e < kend) ? p[(int64_t)row * s_row + (int64_t)(k + e) * s_k]
-                                                                  : from_f32<T>(0.f);
-                }
-            }
-        } else {
-            // block b = wave*4 + i covers 8 row-vectors x 8 k; blocks tile (128/VEC/8) x (BK/8)
-            constexpr int JG = BM / VEC / 8;
-            const int jc_lo = tid & 7, kk = (tid >> 3) & 7, w = tid >> 6;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int b = w * 4 + i;
-                const int jc = (b % JG) * 8 + jc_lo;
-                const int k = k0 + (b / JG) * 8 + kk;
-                const int row = row0 + jc * VEC;
-                if (k < kend && row + VEC <= nrows) {
-                    r[i] = *reinterpret_cast<const Pack<T, VEC>*>(p + (int64_t)k * s_k + row);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e)
-                        r[i].v[e] = (k < kend && row + e < nrows) ? p[(int64_t)k * s_k + row + e] : from_f32<T>(0.f);
-                }
-            }
-        }
-    }
-
-    __device__ __forceinline__ void store(char* __restrict__ lds, int tid) const {
-        if constexpr (MODE == KMAJOR || MODE == GENERIC) {
-            const int c = tid & 7;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = (tid >> 3) + 32 * i;
-                *reinterpret_cast<Pack<T, VEC>*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
-            }
-        } else {
-            constexpr int JG = BM / VEC / 8;
-            const int jc_lo = tid & 7, kk = (tid >> 3) & 7, w = tid >> 6;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int b = w * 4 + i;
-                const int jc = (b % JG) * 8 + jc_lo;
-                const int kb = ((b / JG) * 8 + kk) * (int)sizeof(T);  // byte offset of k inside the row
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const int row = jc * VEC + e;
-                    *reinterpret_cast<T*>(lds + row * BKB + (((kb >> 4) ^ sw(row)) << 4) + (kb & 15)) = r[i].v[e];
-                }
-            }
-        }
-    }
-};
-
-template <typename T>
-__device__ __forceinline__ typename Frag<T>::type read_frag(const char* __restrict__ lds, int row, int q) {
-    return *reinterpret_cast<const typename Frag<T>::type*>(lds + row * BKB + ((q ^ sw(row)) << 4));
-}
+constexpr int BM = 256, BN = 192;       // C tile (rows from A, columns from B)
+constexpr int GEMM_THREADS = 512;
+constexpr int WAVES_N = 2;              // 4 x 2 wavefronts, each 64 rows x 96 columns
+constexpr int TM = 2, TN = 3;           // 32x32 MFMA tiles per wavefront
+constexpr int STAGE_PITCH = 32 * 4 + 16;  // bytes per staged fp32 row of a 64x32 slab
 
 struct GemmArgs {
     const void* a;
@@ -145,17 +49,18 @@ struct GemmArgs {
 };
 
 template <typename T, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
-    // 64 KiB of operand tiles; the epilogue reuses it for 4 staged wave tiles (68 KiB)
-    constexpr int SMEM_BYTES = 4 * 64 * STAGE_PITCH > 2 * (BM + BN) * BKB ? 4 * 64 * STAGE_PITCH : 2 * (BM + BN) * BKB;
+    constexpr int TILE_BYTES = 2 * (BM + BN) * BKB;             // 112 KiB of operand panels
+    constexpr int STAGE_BYTES = (GEMM_THREADS / 64) * 64 * STAGE_PITCH;
+    constexpr int SMEM_BYTES = STAGE_BYTES > TILE_BYTES ? STAGE_BYTES : TILE_BYTES;
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
     auto sA = [&](int p) -> char* { return smem + p * (BM * BKB); };
     auto sB = [&](int p) -> char* { return smem + 2 * BM * BKB + p * (BN * BKB); };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;     // wave position in the 2x2 grid
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int lr = lane & 31, lg = lane >> 5;
 
     // ---- workgroup -> tile ---------------------------------------------------------
@@ -182,109 +87,131 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_kernel(const GemmArgs g)
     const T* A = (const T*)g.a;
     const T* B = (const T*)g.b;
 
-    f32x16 acc[2][2];  // [tn][tm]
+    f32x16 acc[TN][TM];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TM; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    TileLoader<T, AMODE> la;
-    TileLoader<T, BMODE> lb;
-    if (nk > 0) {
-        la.load(A, g.a_row, g.a_k, row0, g.n, kbeg, kend, tid);
-        lb.load(B, g.b_row, g.b_k, col0, g.m, kbeg, kend, tid);
+    // A run of K panels [kt0, kt1): FAST = straight-line vector loads (interior tile, whole
+    // panels), otherwise the element-wise edge loader.
+    auto run = [&](auto fast_tag, int kt0, int kt1) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        if (kt0 >= kt1) return;
+        TileLoader<T, AMODE, BM, GEMM_THREADS> la;
+        TileLoader<T, BMODE, BN, GEMM_THREADS> lb;
+        auto fetch = [&](int kt) {
+            const int k0 = kbeg + kt * BK;
+            if constexpr (FAST) {
+                la.load_fast(A, g.a_row, g.a_k, row0, k0, tid);
+                lb.load_fast(B, g.b_row, g.b_k, col0, k0, tid);
+            } else {
+                la.load_edge(A, g.a_row, g.a_k, row0, g.n, k0, kend, tid);
+                lb.load_edge(B, g.b_row, g.b_k, col0, g.m, k0, kend, tid);
+            }
+        };
+        fetch(kt0);
         la.store(sA(0), tid);
         lb.store(sB(0), tid);
-    }
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const int p = kt & 1;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            la.load(A, g.a_row, g.a_k, row0, g.n, kbeg + (kt + 1) * BK, kend, tid);
-            lb.load(B, g.b_row, g.b_k, col0, g.m, kbeg + (kt + 1) * BK, kend, tid);
-        }
-        const char* cA = sA(p);
-        const char* cB = sB(p);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int q = c * 2 + lg;
-            typename Frag<T>::type fa[2], fb[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                fa[t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q);  // C rows   -> MFMA B operand
-                fb[t] = read_frag<T>(cB, wn * 64 + t * 32 + lr, q);  // C columns-> MFMA A operand
-            }
-#pragma unroll
-            for (int tn = 0; tn < 2; ++tn)
-#pragma unroll
-                for (int tm = 0; tm < 2; ++tm) mma_chunk(acc[tn][tm], fb[tn], fa[tm]);
-        }
-        if (more) {
-            la.store(sA(p ^ 1), tid);
-            lb.store(sB(p ^ 1), tid);
-        }
         __syncthreads();
+        for (int kt = kt0; kt < kt1; ++kt) {
+            const int p = (kt - kt0) & 1;
+            const bool more = kt + 1 < kt1;
+            if (more) fetch(kt + 1);
+            const char* cA = sA(p);
+            const char* cB = sB(p);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int q = c * 2 + lg;
+                typename Frag<T>::type fa[TM], fb[TN];
+#pragma unroll
+                for (int t = 0; t < TM; ++t) fa[t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q);  // C rows    -> MFMA B
+#pragma unroll
+                for (int t = 0; t < TN; ++t) fb[t] = read_frag<T>(cB, wn * 96 + t * 32 + lr, q);  // C columns -> MFMA A
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm) mma_chunk(acc[tn][tm], fb[tn], fa[tm]);
+            }
+            if (more) {
+                la.store(sA(p ^ 1), tid);
+                lb.store(sB(p ^ 1), tid);
+            }
+            __syncthreads();
+        }
+    };
+    constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
+    const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
+    const int nk_full = (kend - kbeg) / BK;  // whole panels
+    if constexpr (VECTOR_OK) {
+        if (interior) {
+            run(std::true_type{}, 0, nk_full);
+            run(std::false_type{}, nk_full, nk);
+        } else {
+            run(std::false_type{}, 0, nk);
+        }
+    } else {
+        run(std::false_type{}, 0, nk);
     }
 
-    // ---- epilogue: stage the wave's 64x64 fp32 tile in LDS, then coalesced row stores --
-    // acc[tn][tm][i] of lane (lr, lg) = C[wm*64 + tm*32 + lr][wn*64 + tn*32 + (i/4)*8 + lg*4 + (i%4)]
+    // ---- epilogue: per 32-column slab, stage the wave's 64x32 fp32 block in LDS, then
+    //      write rows back with contiguous stores.
+    // acc[tn][tm][i] of lane (lr, lg) = C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)]
     char* stage = smem + wave * (64 * STAGE_PITCH);
+    const int cc4 = (lane & 7) * 4;  // 4 consecutive columns of the slab
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn)
+    for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
+        for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 f32x4 v = {acc[tn][tm][i4 * 4 + 0], acc[tn][tm][i4 * 4 + 1], acc[tn][tm][i4 * 4 + 2],
                            acc[tn][tm][i4 * 4 + 3]};
-                const int r = tm * 32 + lr, cc = tn * 32 + i4 * 8 + lg * 4;
-                *reinterpret_cast<f32x4*>(stage + r * STAGE_PITCH + cc * 4) = v;
+                *reinterpret_cast<f32x4*>(stage + (tm * 32 + lr) * STAGE_PITCH + (i4 * 8 + lg * 4) * 4) = v;
             }
-    __syncthreads();
-
-    const int cc4 = (lane & 15) * 4;          // 4 consecutive columns
-    const int gcol = col0 + wn * 64 + cc4;
-    float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-    if (g.epilogue != PTJ_EPI_NONE && g.partial == nullptr) {
+        __syncthreads();
+        const int gcol = col0 + wn * 96 + tn * 32 + cc4;
+        float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (g.epilogue != PTJ_EPI_NONE && g.partial == nullptr) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (gcol + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol + e]);
-    }
+            for (int e = 0; e < 4; ++e)
+                if (gcol + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol + e]);
+        }
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-        const int r = (lane >> 4) + 4 * it;
-        const int grow = row0 + wm * 64 + r;
-        f32x4 v = *reinterpret_cast<const f32x4*>(stage + r * STAGE_PITCH + cc4 * 4);
-        if (grow >= g.n || gcol >= g.m) continue;
-        if (g.partial != nullptr) {
-            float* dst = g.partial + ((int64_t)blockIdx.z * g.n + grow) * g.m + gcol;
-            if (gcol + 4 <= g.m && (((uintptr_t)dst & 15) == 0)) {
-                *reinterpret_cast<f32x4*>(dst) = v;
+        for (int it = 0; it < 8; ++it) {
+            const int r = (lane >> 3) + 8 * it;
+            const int grow = row0 + wm * 64 + r;
+            f32x4 v = *reinterpret_cast<const f32x4*>(stage + r * STAGE_PITCH + cc4 * 4);
+            if (grow >= g.n || gcol >= g.m) continue;
+            if (g.partial != nullptr) {
+                float* dst = g.partial + ((int64_t)blockIdx.z * g.n + grow) * g.m + gcol;
+                if (gcol + 4 <= g.m && (((uintptr_t)dst & 15) == 0)) {
+                    *reinterpret_cast<f32x4*>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gcol + e < g.m) dst[e] = v[e];
+                }
+                continue;
+            }
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = v[e] + bias4[e];
+                if (g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
+            }
+            T* dst = (T*)g.c + (int64_t)grow * g.c_rs + gcol;
+            if (gcol + 4 <= g.m && (((uintptr_t)dst & (4 * sizeof(T) - 1)) == 0)) {
+                store_vec<T, 4>(dst, o);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (gcol + e < g.m) dst[e] = v[e];
+                    if (gcol + e < g.m) dst[e] = from_f32<T>(o[e]);
             }
-            continue;
         }
-        float o[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            o[e] = v[e] + bias4[e];
-            if (g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
-        }
-        T* dst = (T*)g.c + (int64_t)grow * g.c_rs + gcol;
-        if (gcol + 4 <= g.m && (((uintptr_t)dst & (4 * sizeof(T) - 1)) == 0)) {
-            store_vec<T, 4>(dst, o);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (gcol + e < g.m) dst[e] = from_f32<T>(o[e]);
-        }
+        __syncthreads();
     }
 }
 
