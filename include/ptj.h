@@ -127,8 +127,9 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
 
 /* ---- attention ----------------------------------------------------------- */
 
-/* Causal flash-attention forward.  q/k/v/o are [BH, T, dh] views with explicit
- * (batch-head, row) strides and unit stride along dh; `mask` is NULL (pure causal:
+/* Causal flash-attention forward.  q/k/v/o are [B, H, T, dh] views with explicit
+ * (batch, head, row) strides and unit stride along dh -- e.g. slices of the
+ * [B*T, H*3*dh] output of one fused QKV product; `mask` is NULL (pure causal:
  * key j visible to query i iff j <= i) or uint8 [B, T, T] (contiguous) that is
  * ANDed with the causal block structure exactly as the reference kernel does
  * (tiles strictly above the diagonal are never visited; model_triton.py:659-661).
@@ -136,32 +137,38 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
  * exp(score - ms)) as fp32 [BH, T].  Dropout (train != 0) keeps probability
  * (i, j) of batch-head g iff tl.rand(seed + g, i + j) > 0.1; train == 0 scales
  * probabilities by 0.9.  Replaces t_scaled_dot_prod_attn_fwd3_k/_t
- * (model_triton.py:616-754).  Requires dh == 64 and T % 64 == 0. */
+ * (model_triton.py:616-754).  ms/ls are contiguous [B*H, T].  Requires dh == 64, T % 64 == 0, 16-byte aligned
+ * pointers and strides that are multiples of 16 bytes.  A non-NULL mask is applied
+ * as (mask AND key <= query): masks must be sub-masks of the causal mask, as the
+ * training path produces them.  `workspace` is needed when train != 0 only
+ * (ptj_attn_workspace_bytes(B, H, T) bytes; the dropout keep bits live there). */
+size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T);
 int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mask,
-                 void* o, float* ms, float* ls,
+                 void* o, float* ms, float* ls, void* workspace, size_t workspace_bytes,
                  int64_t B, int64_t H, int64_t T, int64_t dh,
-                 int64_t q_bh_stride, int64_t q_row_stride,
-                 int64_t k_bh_stride, int64_t k_row_stride,
-                 int64_t v_bh_stride, int64_t v_row_stride,
-                 int64_t o_bh_stride, int64_t o_row_stride,
+                 int64_t q_b_stride, int64_t q_h_stride, int64_t q_row_stride,
+                 int64_t k_b_stride, int64_t k_h_stride, int64_t k_row_stride,
+                 int64_t v_b_stride, int64_t v_h_stride, int64_t v_row_stride,
+                 int64_t o_b_stride, int64_t o_h_stride, int64_t o_row_stride,
                  int train, int64_t seed, int dtype, void* stream);
 
 /* Flash-attention backward with P recomputed from (ms, ls).  Outputs dq/dk/dv
  * [BH, T, dh] with explicit strides.  Deterministic: dK/dV and dQ are produced by
- * two passes, no atomics.  Replaces t_scaled_dot_prod_attn_bkwd3_k/_t
- * (model_triton.py:829-1003). */
+ * two passes, no atomics.  `workspace` (always required here) holds
+ * ptj_attn_workspace_bytes(B, H, T) bytes.  Replaces
+ * t_scaled_dot_prod_attn_bkwd3_k/_t (model_triton.py:829-1003). */
 int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o,
                  const float* ms, const float* ls, const uint8_t* mask,
-                 void* dq, void* dk, void* dv,
+                 void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes,
                  int64_t B, int64_t H, int64_t T, int64_t dh,
-                 int64_t do_bh_stride, int64_t do_row_stride,
-                 int64_t q_bh_stride, int64_t q_row_stride,
-                 int64_t k_bh_stride, int64_t k_row_stride,
-                 int64_t v_bh_stride, int64_t v_row_stride,
-                 int64_t o_bh_stride, int64_t o_row_stride,
-                 int64_t dq_bh_stride, int64_t dq_row_stride,
-                 int64_t dk_bh_stride, int64_t dk_row_stride,
-                 int64_t dv_bh_stride, int64_t dv_row_stride,
+                 int64_t do_b_stride, int64_t do_h_stride, int64_t do_row_stride,
+                 int64_t q_b_stride, int64_t q_h_stride, int64_t q_row_stride,
+                 int64_t k_b_stride, int64_t k_h_stride, int64_t k_row_stride,
+                 int64_t v_b_stride, int64_t v_h_stride, int64_t v_row_stride,
+                 int64_t o_b_stride, int64_t o_h_stride, int64_t o_row_stride,
+                 int64_t dq_b_stride, int64_t dq_h_stride, int64_t dq_row_stride,
+                 int64_t dk_b_stride, int64_t dk_h_stride, int64_t dk_row_stride,
+                 int64_t dv_b_stride, int64_t dv_h_stride, int64_t dv_row_stride,
                  int train, int64_t seed, int dtype, void* stream);
 
 #ifdef __cplusplus

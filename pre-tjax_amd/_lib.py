@@ -34,8 +34,9 @@ SIGNATURES = {
     "ptj_ce_fwd_bwd": (_int, [_p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "ptj_gemm": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p, _sz, _int, _p]),
-    "ptj_attn_fwd": (_int, [_p, _p, _p, _p, _p, _p, _p] + [_i64] * 12 + [_int, _i64, _int, _p]),
-    "ptj_attn_bwd": (_int, [_p] * 11 + [_i64] * 20 + [_int, _i64, _int, _p]),
+    "ptj_attn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "ptj_attn_fwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz] + [_i64] * 16 + [_int, _i64, _int, _p]),
+    "ptj_attn_bwd": (_int, [_p] * 11 + [_p, _sz] + [_i64] * 28 + [_int, _i64, _int, _p]),
 }
 
 _lib = None

@@ -1,0 +1,730 @@
+// Causal flash attention for gfx950, head dimension 64: forward, and a backward that
+// recomputes P from the saved row max / row sum-exp.
+//
+// Layout trick shared by the three MFMA kernels: scores are produced TRANSPOSED.  With
+// 32x32 MFMA tiles, D[m][n] of lane l sits at n = l & 31, m = 8*(i/4) + 4*(l>>5) + i%4
+// (register i).  Forward and the dQ pass compute S^T = K Q^T, so a lane owns ONE query
+// (n) and 16 keys per 32-key tile (m): row max / row sum / rescaling are per-lane
+// scalars (one cross-lane exchange with lane^32), and the probabilities are already in
+// MFMA B-operand position for O^T = V^T P^T (contraction over keys, which live in the
+// lane's registers), so P never travels through LDS.  The dK/dV pass computes S = Q K^T
+// with the same trick mirrored: a lane owns one key, dV^T = dO^T P and dK^T = Q^T dS.
+// The operand that must be read "across" its memory layout (V^T, K^T, Q^T, dO^T: row
+// index d, contraction along keys / queries) is transposed once while it is written to
+// LDS (MNMAJOR panel loader) and shared by the four wavefronts.
+//
+// Softmax is evaluated in base 2 (scores pre-multiplied by log2(e)/sqrt(dh)); the saved
+// statistics `ms` are converted back to natural units.  Masked scores take the
+// reference's fill value -1e9 (not -inf), including its behaviour on fully masked rows.
+//
+// Dropout on the probabilities: element (q, k) of batch-head g is kept iff
+// philox(seed + g, q + k) passes the threshold -- the offset depends on q + k only, so
+// one line of 2T keep bits per batch-head is generated once (attn_keepbits_kernel) and
+// every kernel extracts a lane's 32-key window from it with one 64-bit shift.
+//
+// The backward is two passes without atomics: (dK, dV) over key tiles, dQ over query
+// tiles; both recompute S and dP.
+#include "common.h"
+#include "mma_tile.h"
+
+namespace {
+
+constexpr int DH = 64;
+constexpr int ATT_THREADS = 256;
+constexpr int PANEL = 64 * BKB;  // bytes of one 64-row LDS panel
+constexpr int MAX_T = 8192;
+constexpr int MAX_BITWORDS = 2 * MAX_T / 32 + 2;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+constexpr float NEG_NAT = -1e9f;
+constexpr float NEG2 = NEG_NAT * LOG2E;
+
+template <typename T> struct AT {
+    static constexpr int ROWB = DH * (int)sizeof(T);   // bytes per q/k/v row: 128 / 256
+    static constexpr int NP = ROWB / BKB;               // panels per 64-element axis: 1 / 2
+    static constexpr int NC = ROWB / 32;                // contraction chunks along d: 4 / 8
+    static constexpr int EPP = BKB / (int)sizeof(T);    // elements per panel row: 64 / 32
+    typedef typename Frag<T>::type F;
+};
+
+struct AttnArgs {
+    const void *q, *k, *v, *o, *d_o;
+    void *out0, *out1;            // fwd: out0 = O.  bwd dkdv: out0 = dK, out1 = dV.  bwd dq: out0 = dQ
+    const uint8_t* mask;          // nullptr = causal by index
+    float *ms, *ls;               // [BH, T]
+    const float* delta;           // [BH, T] rowsum(dO * O)  (backward)
+    const uint32_t* keepbits;     // [BH, bitwords]  (train)
+    int B, H, T, bitwords;
+    // element strides: batch, head, row (the head dimension itself has unit stride)
+    int64_t q_bs, q_hs, q_rs, k_bs, k_hs, k_rs, v_bs, v_hs, v_rs, o_bs, o_hs, o_rs, do_bs, do_hs, do_rs;
+    int64_t out0_bs, out0_hs, out0_rs, out1_bs, out1_hs, out1_rs;
+    int train;
+    float scale;                  // 1/sqrt(dh)
+};
+
+// ---- small device helpers -----------------------------------------------------------
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// The 16-byte operand pieces of one 64-element row held in registers (lane half lg).
+template <typename T>
+__device__ __forceinline__ void load_row_frags(typename AT<T>::F (&f)[AT<T>::NC], const T* __restrict__ row, int lg) {
+#pragma unroll
+    for (int c = 0; c < AT<T>::NC; ++c)
+        f[c] = *reinterpret_cast<const typename AT<T>::F*>(reinterpret_cast<const char*>(row) + c * 32 + lg * 16);
+}
+
+// s[j] += panel_rows(j*32 + lr) x register_rows : panel rows become MFMA rows (m), the
+// lane's register row the MFMA column (n); contraction over the 64-element axis d.
+template <typename T>
+__device__ __forceinline__ void rows_x_frags(f32x16 (&s)[2], const char* __restrict__ panels,
+                                             const typename AT<T>::F (&f)[AT<T>::NC], int lr, int lg) {
+#pragma unroll
+    for (int c = 0; c < AT<T>::NC; ++c) {
+        const char* pp = panels + (c / 4) * PANEL;
+        const int q = (c % 4) * 2 + lg;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            typename AT<T>::F a = read_frag<T>(pp, j * 32 + lr, q);
+            mma_chunk(s[j], a, f[c]);
+        }
+    }
+}
+
+// o[t] += transposed_panel_rows(t*32 + lr) x p : contraction over the 64 positions whose
+// values p[j][i] the lane holds in accumulator order (position = j*32 + 8*(i/4) + 4*lg + i%4).
+__device__ __forceinline__ void tp_x_regs(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[2][16],
+                                          int lr, int lg, bf16) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            bf16x8 b;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[e] = (bf16)p[j][8 * h + e];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int row = t * 32 + lr;
+                const char* rp = panels + row * BKB + lg * 8;
+                const bf16x4 lo = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h) ^ sw(row)) << 4));
+                const bf16x4 hi = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h + 1) ^ sw(row)) << 4));
+                const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, o[t], 0, 0, 0);
+            }
+        }
+}
+__device__ __forceinline__ void tp_x_regs(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[2][16],
+                                          int lr, int lg, float) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const char* pp = panels + j * PANEL;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const f32x4 v = read_frag<float>(pp, t * 32 + lr, 2 * a + lg);
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[b], p[j][4 * a + b], o[t], 0, 0, 0);
+            }
+    }
+}
+
+// 32 keep bits starting at bit `ob` of the batch-head's bit line (LDS copy).
+__device__ __forceinline__ uint32_t keep_window(const uint32_t* __restrict__ sbits, int ob) {
+    const int w = ob >> 5, sh = ob & 31;
+    const uint64_t v = ((uint64_t)sbits[w + 1] << 32) | sbits[w];
+    return (uint32_t)(v >> sh);
+}
+
+// Store the transposed accumulators acc[t][i] (row = the lane's position `pos`, column
+// d = t*32 + 8*(i/4) + 4*lg + i%4) scaled by `f` as rows of a [.., 64] tensor.
+template <typename T>
+__device__ __forceinline__ void store_rows(T* __restrict__ row, const f32x16 (&acc)[2], float f, int lg) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            float v[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) v[b] = acc[t][4 * a + b] * f;
+            store_vec<T, 4>(row + t * 32 + a * 8 + lg * 4, v);
+        }
+}
+
+// ---- keep-bit line per batch-head ---------------------------------------------------
+__global__ __launch_bounds__(256) void attn_keepbits_kernel(uint32_t* __restrict__ bits, int bitwords, uint64_t seed) {
+    const int bh = blockIdx.y;
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    const uint64_t s = seed + (uint64_t)bh;
+    const bool keep = philox_keep((uint32_t)o, (uint32_t)s, (uint32_t)(s >> 32));
+    const uint64_t m = __ballot(keep);
+    if ((threadIdx.x & 63) == 0) {
+        const int w = o >> 5;
+        uint32_t* dst = bits + (int64_t)bh * bitwords;
+        if (w < bitwords) dst[w] = (uint32_t)m;
+        if (w + 1 < bitwords) dst[w + 1] = (uint32_t)(m >> 32);
+    }
+}
+
+// ---- delta[bh, q] = sum_d dO[q,d] * O[q,d] -------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
+                                                          float* __restrict__ delta, int T_, int H_,
+                                                          int64_t do_bs, int64_t do_hs, int64_t do_rs, int64_t o_bs,
+                                                          int64_t o_hs, int64_t o_rs) {
+    const int bh = blockIdx.y;
+    const int64_t do_off = (bh / H_) * do_bs + (bh % H_) * do_hs, o_off = (bh / H_) * o_bs + (bh % H_) * o_hs;
+    const int row = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const int c = (threadIdx.x & 7) * 8;
+    float s = 0.f;
+    if (row < T_) {
+        const T* pa = d_o + do_off + (int64_t)row * do_rs + c;
+        const T* pb = o + o_off + (int64_t)row * o_rs + c;
+        constexpr int V = VecOf<T>::N;
+#pragma unroll
+        for (int h = 0; h < 8 / V; ++h) {
+            float x[V], y[V];
+            load_vec<T, V>(pa + h * V, x);
+            load_vec<T, V>(pb + h * V, y);
+#pragma unroll
+            for (int e = 0; e < V; ++e) s += x[e] * y[e];
+        }
+    }
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    s += __shfl_xor(s, 4, 64);
+    if ((threadIdx.x & 7) == 0 && row < T_) delta[(int64_t)bh * T_ + row] = s;
+}
+
+// ---- forward -------------------------------------------------------------------------
+// grid (ceil(T/128), B*H); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
+template <typename T>
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
+    typedef AT<T> X;
+    constexpr int STAGE = 2 * X::NP * PANEL;  // K panels then V^T panels
+    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    __shared__ uint32_t sbits[MAX_BITWORDS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128;   // heavy (late) query tiles first
+    const int qw0 = q0 + wave * 32;
+    const int query = qw0 + lr;
+    const int qrow = query < a.T ? query : a.T - 1;
+
+    const T* Qb = (const T*)a.q + bidx * a.q_bs + hidx * a.q_hs;
+    const T* Kb = (const T*)a.k + bidx * a.k_bs + hidx * a.k_hs;
+    const T* Vb = (const T*)a.v + bidx * a.v_bs + hidx * a.v_hs;
+
+    typename X::F qf[X::NC];
+    load_row_frags<T>(qf, Qb + (int64_t)qrow * a.q_rs, lg);
+
+    int nkt = (q0 + 128) / 64;
+    if (nkt > a.T / 64) nkt = a.T / 64;
+
+    TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lv[X::NP];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lk[p].load_fast(Kb, a.k_rs, 1, kt * 64, p * X::EPP, tid);
+            lv[p].load_fast(Vb, 1, a.v_rs, 0, kt * 64 + p * X::EPP, tid);
+        }
+    };
+    auto stash = [&](int st) {
+        char* base = smem + st * STAGE;
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lk[p].store(base + p * PANEL, tid);
+            lv[p].store(base + (X::NP + p) * PANEL, tid);
+        }
+    };
+
+    fetch(0);
+    if (a.train) {
+        const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
+        for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
+    }
+    stash(0);
+    __syncthreads();
+
+    const float sc = a.scale * LOG2E;
+    float m_run = NEG2, l_run = 0.f;
+    f32x16 o[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+
+    for (int kt = 0; kt < nkt; ++kt) {
+        const int st = kt & 1;
+        const bool more = kt + 1 < nkt;
+        if (more) fetch(kt + 1);
+        const int key0 = kt * 64;
+        if (key0 <= qw0 + 31) {   // some key of this tile is visible to some query of the wave
+            const char* kp = smem + st * STAGE;
+            const char* vp = kp + X::NP * PANEL;
+            f32x16 s[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[j][e] = 0.f;
+            rows_x_frags<T>(s, kp, qf, lr, lg);
+
+            float p[2][16];
+            const bool diag = key0 + 63 > qw0;
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
+                    uint32_t m4 = 0x01010101u;
+                    if (a.mask) m4 = *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        float v = s[j][g4 * 4 + b] * sc;
+                        bool ok = ((m4 >> (8 * b)) & 0xff) != 0;
+                        if (diag) ok = ok && (kb + b <= query);
+                        v = ok ? v : NEG2;
+                        p[j][g4 * 4 + b] = v;
+                        tmax = fmaxf(tmax, v);
+                    }
+                }
+            tmax = fmaxf(tmax, xor32(tmax));
+            const float m_new = fmaxf(m_run, tmax);
+            const float alpha = fast_exp2(m_run - m_new);
+            float lsum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float e = fast_exp2(p[j][i] - m_new);
+                    p[j][i] = e;
+                    lsum += e;
+                }
+            lsum += xor32(lsum);
+            l_run = l_run * alpha + lsum;
+            m_run = m_new;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+            if (a.train) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        p[j][i] = ((w >> ((i >> 2) * 8 + (i & 3))) & 1u) ? p[j][i] : 0.f;
+                }
+            }
+            tp_x_regs(o, vp, p, lr, lg, T());
+        }
+        if (more) stash(st ^ 1);
+        __syncthreads();
+    }
+
+    if (query < a.T) {
+        const float f = (a.train ? 1.0f : 0.9f) / l_run;
+        store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, o, f, lg);
+        if (lg == 0) {
+            a.ms[(int64_t)bh * a.T + query] = m_run == NEG2 ? NEG_NAT : m_run * LN2;
+            a.ls[(int64_t)bh * a.T + query] = l_run;
+        }
+    }
+}
+
+// Shared by both backward passes: probability and score-gradient of one element.
+//   v   : scaled score in log2 units (already masked to NEG2 where invisible)
+//   dpv : dP element;  keep: dropout keep bit (train) -- eval scales by 0.9
+// returns P (pre-dropout); writes pd (post-dropout P) and ds (unscaled dS).
+__device__ __forceinline__ void softmax_bwd_elem(float v, float dpv, bool visible, bool keep, int train, float m2,
+                                                 float linv, float delta, float& pd, float& ds) {
+    const float p = fast_exp2(v - m2) * linv;
+    if (train) {
+        pd = keep ? p : 0.f;
+        dpv = keep ? dpv : 0.f;
+    } else {
+        pd = 0.9f * p;
+        dpv = 0.9f * dpv;
+    }
+    ds = visible ? p * (dpv - delta) : 0.f;
+}
+
+// ---- backward pass 1: dK, dV ------------------------------------------------------------
+// grid (ceil(T/128), B*H); wave w owns keys key0 + 32w .. +31 (lane = key); query tiles of 64.
+template <typename T>
+__global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+    typedef AT<T> X;
+    constexpr int STAGE = 4 * X::NP * PANEL;  // Q, dO, Q^T, dO^T
+    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    __shared__ __attribute__((aligned(16))) float sstat[2][3][64];  // m2, 1/l, delta per stage
+    __shared__ uint32_t sbits[MAX_BITWORDS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
+    const int key0 = blockIdx.x * 128;
+    const int kw0 = key0 + wave * 32;
+    const int key = kw0 + lr;
+    const int krow = key < a.T ? key : a.T - 1;
+
+    const T* Qb = (const T*)a.q + bidx * a.q_bs + hidx * a.q_hs;
+    const T* Kb = (const T*)a.k + bidx * a.k_bs + hidx * a.k_hs;
+    const T* Vb = (const T*)a.v + bidx * a.v_bs + hidx * a.v_hs;
+    const T* dOb = (const T*)a.d_o + bidx * a.do_bs + hidx * a.do_hs;
+
+    typename X::F kf[X::NC], vf[X::NC];
+    load_row_frags<T>(kf, Kb + (int64_t)krow * a.k_rs, lg);
+    load_row_frags<T>(vf, Vb + (int64_t)krow * a.v_rs, lg);
+
+    const int qt0 = key0 / 64, nqt = a.T / 64;
+
+    TileLoader<T, KMAJOR, 64, ATT_THREADS> lq[X::NP], ld[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lqt[X::NP], ldt[X::NP];
+    float st_m = 0.f, st_l = 1.f, st_d = 0.f;
+    auto fetch = [&](int qt) {
+        const int q0 = qt * 64;
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lq[p].load_fast(Qb, a.q_rs, 1, q0, p * X::EPP, tid);
+            ld[p].load_fast(dOb, a.do_rs, 1, q0, p * X::EPP, tid);
+            lqt[p].load_fast(Qb, 1, a.q_rs, 0, q0 + p * X::EPP, tid);
+            ldt[p].load_fast(dOb, 1, a.do_rs, 0, q0 + p * X::EPP, tid);
+        }
+        if (tid < 64) {
+            const int64_t i = (int64_t)bh * a.T + q0 + tid;
+            st_m = a.ms[i];
+            st_l = a.ls[i];
+            st_d = a.delta[i];
+        }
+    };
+    auto stash = [&](int st) {
+        char* base = smem + st * STAGE;
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lq[p].store(base + p * PANEL, tid);
+            ld[p].store(base + (X::NP + p) * PANEL, tid);
+            lqt[p].store(base + (2 * X::NP + p) * PANEL, tid);
+            ldt[p].store(base + (3 * X::NP + p) * PANEL, tid);
+        }
+        if (tid < 64) {
+            sstat[st][0][tid] = st_m * LOG2E;
+            sstat[st][1][tid] = 1.0f / st_l;
+            sstat[st][2][tid] = st_d;
+        }
+    };
+
+    f32x16 dk[2], dv[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dk[t][e] = dv[t][e] = 0.f;
+
+    if (qt0 < nqt) {
+        fetch(qt0);
+        if (a.train) {
+            const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
+            for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
+        }
+        stash(0);
+    }
+    __syncthreads();
+
+    const float sc = a.scale * LOG2E;
+    for (int qt = qt0; qt < nqt; ++qt) {
+        const int st = (qt - qt0) & 1;
+        const bool more = qt + 1 < nqt;
+        if (more) fetch(qt + 1);
+        const int q0 = qt * 64;
+        if (q0 + 63 >= kw0) {   // some query of the tile sees some key of the wave
+            const char* base = smem + st * STAGE;
+            f32x16 s[2], dp[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[j][e] = dp[j][e] = 0.f;
+            rows_x_frags<T>(s, base, kf, lr, lg);                          // S  [query][key]
+            rows_x_frags<T>(dp, base + X::NP * PANEL, vf, lr, lg);         // dP [query][key]
+
+            float pd[2][16], ds[2][16];
+            const bool diag = q0 < kw0 + 31;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t w = 0xffffffffu;
+                if (a.train) w = keep_window(sbits, key + q0 + j * 32 + lg * 4);
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int qi = j * 32 + g4 * 8 + lg * 4;  // first of 4 consecutive queries (tile-relative)
+                    const f32x4 m4 = *reinterpret_cast<const f32x4*>(&sstat[st][0][qi]);
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[st][1][qi]);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[st][2][qi]);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const int i = g4 * 4 + b;
+                        const int qq = q0 + qi + b;
+                        bool ok = true;
+                        if (a.mask) ok = a.mask[((int64_t)bidx * a.T + qq) * a.T + krow] != 0;
+                        if (diag) ok = ok && (key <= qq);
+                        const float v = ok ? s[j][i] * sc : NEG2;
+                        softmax_bwd_elem(v, dp[j][i], ok, (w >> (g4 * 8 + b)) & 1u, a.train, m4[b], l4[b], d4[b],
+                                         pd[j][i], ds[j][i]);
+                    }
+                }
+            }
+            tp_x_regs(dv, base + 3 * X::NP * PANEL, pd, lr, lg, T());      // dV^T += dO^T P
+            tp_x_regs(dk, base + 2 * X::NP * PANEL, ds, lr, lg, T());      // dK^T += Q^T dS
+        }
+        if (more) stash(st ^ 1);
+        __syncthreads();
+    }
+
+    if (key < a.T) {
+        store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)key * a.out0_rs, dk, a.scale, lg);
+        store_rows<T>((T*)a.out1 + bidx * a.out1_bs + hidx * a.out1_hs + (int64_t)key * a.out1_rs, dv, 1.0f, lg);
+    }
+}
+
+// ---- backward pass 2: dQ ----------------------------------------------------------------
+// Same geometry as the forward (lane = query, key tiles of 64).
+template <typename T>
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
+    typedef AT<T> X;
+    constexpr int STAGE = 3 * X::NP * PANEL;  // K, V, K^T
+    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    __shared__ uint32_t sbits[MAX_BITWORDS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128;
+    const int qw0 = q0 + wave * 32;
+    const int query = qw0 + lr;
+    const int qrow = query < a.T ? query : a.T - 1;
+
+    const T* Qb = (const T*)a.q + bidx * a.q_bs + hidx * a.q_hs;
+    const T* Kb = (const T*)a.k + bidx * a.k_bs + hidx * a.k_hs;
+    const T* Vb = (const T*)a.v + bidx * a.v_bs + hidx * a.v_hs;
+    const T* dOb = (const T*)a.d_o + bidx * a.do_bs + hidx * a.do_hs;
+
+    typename X::F qf[X::NC], dof[X::NC];
+    load_row_frags<T>(qf, Qb + (int64_t)qrow * a.q_rs, lg);
+    load_row_frags<T>(dof, dOb + (int64_t)qrow * a.do_rs, lg);
+    const int64_t si = (int64_t)bh * a.T + qrow;
+    const float m2 = a.ms[si] * LOG2E, linv = 1.0f / a.ls[si], delta = a.delta[si];
+
+    int nkt = (q0 + 128) / 64;
+    if (nkt > a.T / 64) nkt = a.T / 64;
+
+    TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP], lv[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lkt[X::NP];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lk[p].load_fast(Kb, a.k_rs, 1, kt * 64, p * X::EPP, tid);
+            lv[p].load_fast(Vb, a.v_rs, 1, kt * 64, p * X::EPP, tid);
+            lkt[p].load_fast(Kb, 1, a.k_rs, 0, kt * 64 + p * X::EPP, tid);
+        }
+    };
+    auto stash = [&](int st) {
+        char* base = smem + st * STAGE;
+#pragma unroll
+        for (int p = 0; p < X::NP; ++p) {
+            lk[p].store(base + p * PANEL, tid);
+            lv[p].store(base + (X::NP + p) * PANEL, tid);
+            lkt[p].store(base + (2 * X::NP + p) * PANEL, tid);
+        }
+    };
+
+    fetch(0);
+    if (a.train) {
+        const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
+        for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
+    }
+    stash(0);
+    __syncthreads();
+
+    const float sc = a.scale * LOG2E;
+    f32x16 dq[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dq[t][e] = 0.f;
+
+    for (int kt = 0; kt < nkt; ++kt) {
+        const int st = kt & 1;
+        const bool more = kt + 1 < nkt;
+        if (more) fetch(kt + 1);
+        const int key0 = kt * 64;
+        if (key0 <= qw0 + 31) {
+            const char* base = smem + st * STAGE;
+            f32x16 s[2], dp[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[j][e] = dp[j][e] = 0.f;
+            rows_x_frags<T>(s, base, qf, lr, lg);                        // S^T  [key][query]
+            rows_x_frags<T>(dp, base + X::NP * PANEL, dof, lr, lg);      // dP^T [key][query]
+
+            float ds[2][16];
+            const bool diag = key0 + 63 > qw0;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t w = 0xffffffffu;
+                if (a.train) w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
+                    uint32_t m4 = 0x01010101u;
+                    if (a.mask) m4 = *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const int i = g4 * 4 + b;
+                        bool ok = ((m4 >> (8 * b)) & 0xff) != 0;
+                        if (diag) ok = ok && (kb + b <= query);
+                        const float v = ok ? s[j][i] * sc : NEG2;
+                        float pd_unused;
+                        softmax_bwd_elem(v, dp[j][i], ok, (w >> (g4 * 8 + b)) & 1u, a.train, m2, linv, delta, pd_unused,
+                                         ds[j][i]);
+                    }
+                }
+            }
+            tp_x_regs(dq, base + 2 * X::NP * PANEL, ds, lr, lg, T());    // dQ^T += K^T dS^T
+        }
+        if (more) stash(st ^ 1);
+        __syncthreads();
+    }
+
+    if (query < a.T) store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, dq, a.scale, lg);
+}
+
+// ---- host side ----------------------------------------------------------------------------
+inline size_t bits_bytes(int64_t BH, int64_t T) { return (size_t)BH * (2 * T / 32 + 2) * sizeof(uint32_t); }
+inline size_t delta_bytes(int64_t BH, int64_t T) { return (size_t)BH * T * sizeof(float); }
+
+int check_common(const char* what, int64_t B, int64_t H, int64_t T, int64_t dh, int dtype,
+                 std::initializer_list<const void*> ptrs, std::initializer_list<int64_t> strides) {
+    if (B < 1 || H < 1) return ptj_set_error(PTJ_ERR_INVALID, "%s: B and H must be positive", what);
+    if (dh != DH) return ptj_set_error(PTJ_ERR_INVALID, "%s: head dimension %lld unsupported (64 only)", what, (long long)dh);
+    if (T < 64 || T % 64 != 0 || T > MAX_T)
+        return ptj_set_error(PTJ_ERR_INVALID, "%s: T=%lld must be a multiple of 64 in [64, %d]", what, (long long)T, MAX_T);
+    if (dtype != PTJ_F32 && dtype != PTJ_BF16) return ptj_set_error(PTJ_ERR_INVALID, "%s: unknown dtype %d", what, dtype);
+    const int vec = dtype == PTJ_BF16 ? 8 : 4;
+    for (const void* p : ptrs)
+        if (!p || !ptj_aligned16(p)) return ptj_set_error(PTJ_ERR_INVALID, "%s: null or not 16-byte aligned pointer", what);
+    for (int64_t s : strides)
+        if (s % vec != 0 || s < 0) return ptj_set_error(PTJ_ERR_INVALID, "%s: strides must be multiples of 16 bytes", what);
+    return PTJ_OK;
+}
+
+int launch_keepbits(uint32_t* bits, int64_t BH, int bitwords, int64_t seed, hipStream_t st) {
+    hipLaunchKernelGGL(attn_keepbits_kernel, dim3((bitwords * 32 + 255) / 256, (unsigned)BH), dim3(256), 0, st, bits,
+                       bitwords, (uint64_t)seed);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T) {
+    if (B < 1 || H < 1 || T < 1) return 0;
+    return bits_bytes(B * H, T) + delta_bytes(B * H, T);
+}
+
+int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, float* ms, float* ls,
+                 void* workspace, size_t workspace_bytes, int64_t B, int64_t H, int64_t T, int64_t dh,
+                 int64_t q_bs, int64_t q_hs, int64_t q_rs, int64_t k_bs, int64_t k_hs, int64_t k_rs,
+                 int64_t v_bs, int64_t v_hs, int64_t v_rs, int64_t o_bs, int64_t o_hs, int64_t o_rs,
+                 int train, int64_t seed, int dtype, void* stream) {
+    int rc = check_common("attn_fwd", B, H, T, dh, dtype, {q, k, v, o},
+                          {q_bs, q_hs, q_rs, k_bs, k_hs, k_rs, v_bs, v_hs, v_rs, o_bs, o_hs, o_rs});
+    if (rc) return rc;
+    PTJ_CHECK_ARG(ms && ls, "attn_fwd: null statistics pointer");
+    PTJ_CHECK_ARG(!mask || (reinterpret_cast<uintptr_t>(mask) & 3) == 0, "attn_fwd: mask must be 4-byte aligned");
+    const int64_t BH = B * H;
+    hipStream_t st = (hipStream_t)stream;
+    AttnArgs a = {};
+    a.q = q; a.k = k; a.v = v; a.out0 = o; a.mask = mask; a.ms = ms; a.ls = ls;
+    a.B = (int)B; a.H = (int)H; a.T = (int)T; a.bitwords = (int)(2 * T / 32 + 2);
+    a.q_bs = q_bs; a.q_hs = q_hs; a.q_rs = q_rs; a.k_bs = k_bs; a.k_hs = k_hs; a.k_rs = k_rs;
+    a.v_bs = v_bs; a.v_hs = v_hs; a.v_rs = v_rs;
+    a.out0_bs = o_bs; a.out0_hs = o_hs; a.out0_rs = o_rs;
+    a.train = train != 0; a.scale = 0.125f;
+    if (a.train) {
+        if (!workspace || workspace_bytes < bits_bytes(BH, T))
+            return ptj_set_error(PTJ_ERR_WORKSPACE, "attn_fwd: workspace %zu < %zu bytes", workspace_bytes, bits_bytes(BH, T));
+        a.keepbits = (const uint32_t*)workspace;
+        rc = launch_keepbits((uint32_t*)workspace, BH, a.bitwords, seed, st);
+        if (rc) return rc;
+    }
+    dim3 grid((unsigned)((T + 127) / 128), (unsigned)BH);
+    if (dtype == PTJ_F32) hipLaunchKernelGGL((attn_fwd_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o, const float* ms,
+                 const float* ls, const uint8_t* mask, void* dq, void* dk, void* dv, void* workspace,
+                 size_t workspace_bytes, int64_t B, int64_t H, int64_t T, int64_t dh,
+                 int64_t do_bs, int64_t do_hs, int64_t do_rs, int64_t q_bs, int64_t q_hs, int64_t q_rs,
+                 int64_t k_bs, int64_t k_hs, int64_t k_rs, int64_t v_bs, int64_t v_hs, int64_t v_rs,
+                 int64_t o_bs, int64_t o_hs, int64_t o_rs, int64_t dq_bs, int64_t dq_hs, int64_t dq_rs,
+                 int64_t dk_bs, int64_t dk_hs, int64_t dk_rs, int64_t dv_bs, int64_t dv_hs, int64_t dv_rs,
+                 int train, int64_t seed, int dtype, void* stream) {
+    int rc = check_common("attn_bwd", B, H, T, dh, dtype, {d_o, q, k, v, o, dq, dk, dv},
+                          {do_bs, do_hs, do_rs, q_bs, q_hs, q_rs, k_bs, k_hs, k_rs, v_bs, v_hs, v_rs, o_bs, o_hs, o_rs,
+                           dq_bs, dq_hs, dq_rs, dk_bs, dk_hs, dk_rs, dv_bs, dv_hs, dv_rs});
+    if (rc) return rc;
+    PTJ_CHECK_ARG(ms && ls, "attn_bwd: null statistics pointer");
+    PTJ_CHECK_ARG(!mask || (reinterpret_cast<uintptr_t>(mask) & 3) == 0, "attn_bwd: mask must be 4-byte aligned");
+    const int64_t BH = B * H;
+    if (!workspace || workspace_bytes < ptj_attn_workspace_bytes(B, H, T))
+        return ptj_set_error(PTJ_ERR_WORKSPACE, "attn_bwd: workspace %zu < %zu bytes", workspace_bytes,
+                             ptj_attn_workspace_bytes(B, H, T));
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t* bits = (uint32_t*)workspace;
+    float* delta = (float*)((char*)workspace + bits_bytes(BH, T));
+    AttnArgs a = {};
+    a.q = q; a.k = k; a.v = v; a.o = o; a.d_o = d_o; a.mask = mask;
+    a.ms = const_cast<float*>(ms); a.ls = const_cast<float*>(ls); a.delta = delta; a.keepbits = bits;
+    a.B = (int)B; a.H = (int)H; a.T = (int)T; a.bitwords = (int)(2 * T / 32 + 2);
+    a.q_bs = q_bs; a.q_hs = q_hs; a.q_rs = q_rs; a.k_bs = k_bs; a.k_hs = k_hs; a.k_rs = k_rs;
+    a.v_bs = v_bs; a.v_hs = v_hs; a.v_rs = v_rs; a.o_bs = o_bs; a.o_hs = o_hs; a.o_rs = o_rs;
+    a.do_bs = do_bs; a.do_hs = do_hs; a.do_rs = do_rs;
+    a.train = train != 0; a.scale = 0.125f;
+    if (a.train) {
+        rc = launch_keepbits(bits, BH, a.bitwords, seed, st);
+        if (rc) return rc;
+    }
+    dim3 dgrid((unsigned)((T + 31) / 32), (unsigned)BH);
+    if (dtype == PTJ_F32)
+        hipLaunchKernelGGL((attn_delta_kernel<float>), dgrid, dim3(256), 0, st, (const float*)d_o, (const float*)o, delta,
+                           (int)T, (int)H, do_bs, do_hs, do_rs, o_bs, o_hs, o_rs);
+    else
+        hipLaunchKernelGGL((attn_delta_kernel<bf16>), dgrid, dim3(256), 0, st, (const bf16*)d_o, (const bf16*)o, delta,
+                           (int)T, (int)H, do_bs, do_hs, do_rs, o_bs, o_hs, o_rs);
+    PTJ_CHECK_LAUNCH();
+    dim3 grid((unsigned)((T + 127) / 128), (unsigned)BH);
+    AttnArgs a1 = a;
+    a1.out0 = dk; a1.out0_bs = dk_bs; a1.out0_hs = dk_hs; a1.out0_rs = dk_rs;
+    a1.out1 = dv; a1.out1_bs = dv_bs; a1.out1_hs = dv_hs; a1.out1_rs = dv_rs;
+    AttnArgs a2 = a;
+    a2.out0 = dq; a2.out0_bs = dq_bs; a2.out0_hs = dq_hs; a2.out0_rs = dq_rs;
+    if (dtype == PTJ_F32) {
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a1);
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a2);
+    } else {
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a1);
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a2);
+    }
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+}  // extern "C"

@@ -231,3 +231,101 @@ def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
     mid = matmul_t(x2, w1.t(), b1, gelu=True)
     out = matmul_t(mid, w2.t(), b2)
     return out.view(shape[:-1] + (w2.shape[0],))
+
+
+# ----------------------------------------------------------------------------------
+# attention  (reference: model_triton.py:706-754 fwd3_t, :951-1003 bkwd3_t)
+# ----------------------------------------------------------------------------------
+_mask_cache = {}
+
+
+def _mask_arg(mask, B, T):
+    """None when `mask` is exactly the causal (lower-triangular) mask -- the kernel then
+    masks by index -- else a contiguous uint8 [B,T,T] tensor.  The comparison reads the
+    mask once per distinct tensor (one host sync) and is cached on (storage, version)."""
+    if mask is None:
+        return None
+    assert mask.shape[-2:] == (T, T), mask.shape
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.device)
+    hit = _mask_cache.get(key)
+    if hit is None:
+        m = mask.expand(B, T, T) if mask.dim() == 3 else mask.reshape(1, T, T).expand(B, T, T)
+        tril = torch.ones(T, T, dtype=torch.bool, device=mask.device).tril_()
+        if bool((m.to(torch.bool) == tril).all()):
+            hit = ("causal", None)
+        else:
+            hit = ("mask", m.to(torch.bool).contiguous().view(torch.uint8))
+        if len(_mask_cache) > 64:
+            _mask_cache.clear()
+        _mask_cache[key] = hit
+    return hit[1]
+
+
+def _bhr(t):
+    """(batch, head, row) element strides of a [B,H,T,dh] view with unit last stride."""
+    assert t.stride(3) == 1, "head dimension must be contiguous"
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def attn_fwd_t(q, k, v, mask, train, seed, out=None):
+    """Flash-attention forward on [B,H,T,dh] *views* (any batch/head/row strides).
+    Returns (O, ms[B,H,T] fp32, ls[B,H,T] fp32).  `out` may be a preallocated view."""
+    require_gpu(q, k, v)
+    B, H, T, dh = q.shape
+    assert k.shape == q.shape and v.shape == q.shape and q.dtype == k.dtype == v.dtype
+    assert T % 64 == 0, "sequence length must be a multiple of 64"
+    if out is None:
+        out = torch.empty((B, H, T, dh), dtype=q.dtype, device=q.device)
+    ms = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
+    ls = torch.empty_like(ms)
+    m = _mask_arg(mask, B, T)
+    ws_bytes = lib().ptj_attn_workspace_bytes(B, H, T) if train else 0
+    ws = _workspace(ws_bytes, q.device, "attn") if train else None
+    check(lib().ptj_attn_fwd(ptr(q), ptr(k), ptr(v), ptr(m), ptr(out), ptr(ms), ptr(ls), ptr(ws), ws_bytes,
+                             B, H, T, dh, *_bhr(q), *_bhr(k), *_bhr(v), *_bhr(out),
+                             int(bool(train)), int(seed if train else 0), dtype_code(q), stream()), "ptj_attn_fwd")
+    return out, ms, ls
+
+
+def attn_bwd_t(d_o, q, k, v, o, ms, ls, mask, train, seed, out=None):
+    """Flash-attention backward on [B,H,T,dh] views; returns (dq, dk, dv) (views of `out`
+    = (dq, dk, dv) when given)."""
+    require_gpu(d_o, q, k, v, o)
+    B, H, T, dh = q.shape
+    if out is None:
+        out = tuple(torch.empty((B, H, T, dh), dtype=q.dtype, device=q.device) for _ in range(3))
+    dq, dk, dv = out
+    m = _mask_arg(mask, B, T)
+    ws_bytes = lib().ptj_attn_workspace_bytes(B, H, T)
+    ws = _workspace(ws_bytes, q.device, "attn")
+    ms = ms.contiguous()
+    ls = ls.contiguous()
+    check(lib().ptj_attn_bwd(ptr(d_o), ptr(q), ptr(k), ptr(v), ptr(o), ptr(ms), ptr(ls), ptr(m), ptr(dq), ptr(dk),
+                             ptr(dv), ptr(ws), ws_bytes, B, H, T, dh, *_bhr(d_o), *_bhr(q), *_bhr(k), *_bhr(v),
+                             *_bhr(o), *_bhr(dq), *_bhr(dk), *_bhr(dv), int(bool(train)),
+                             int(seed if train else 0), dtype_code(q), stream()), "ptj_attn_bwd")
+    return dq, dk, dv
+
+
+def _aligned_view(t):
+    """Kernel operand requirements: 16-byte aligned base, strides multiple of 16 bytes."""
+    vec = 16 // t.element_size()
+    if t.stride(3) != 1 or t.data_ptr() % 16 or any(s % vec for s in t.stride()[:3]):
+        return t.contiguous()
+    return t
+
+
+def t_scaled_dot_prod_attn_fwd3_t(qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
+    """qkv [B,H,3,T,dh], mask [B,T,T] bool -> (O [B,H,T,dh], [ms, ls, O])."""
+    q, k, v = (_aligned_view(t) for t in torch.unbind(qkv, dim=2))
+    if train:
+        assert p_gen_aux is not None
+    o, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux)
+    return o, [ms, ls, o]
+
+
+def t_scaled_dot_prod_attn_bkwd3_t(dloss_dx, acts, qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
+    """-> (dq, dk, dv), each [B,H,T,dh]."""
+    q, k, v = (_aligned_view(t) for t in torch.unbind(qkv, dim=2))
+    ms, ls, o = acts
+    return attn_bwd_t(_aligned_view(dloss_dx), q, k, v, _aligned_view(o), ms, ls, mask, train, p_gen_aux)

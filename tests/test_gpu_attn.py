@@ -1,0 +1,132 @@
+"""GPU parity of the flash-attention kernels (through the C ABI) against the fp64 oracle on
+the same (dtype-rounded) inputs.  Tolerances: fp32 rtol 1e-5 relative to the tensor's scale
+(atol = 1e-5 * max|want|) ; bf16 2e-2 likewise.  Dropout masks are exercised through the
+train-mode output (the oracle applies the Philox keep mask of the reference kernel)."""
+import pytest
+import torch
+
+from oracle import ops
+from util import DTYPES, f64, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def close(got, want, dtype, what):
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    scale = want.abs().max().item()
+    err = (f64(got) - want).abs().max().item()
+    assert err <= tol * max(scale, 1e-30), "%s: max err %.3e vs scale %.3e (tol %g)" % (what, err, scale, tol)
+
+
+def make(B, H, T, dtype, seed=0):
+    g = gen(seed)
+    qkv = randn(g, B, H, 3, T, 64, dtype=dtype)
+    dO = randn(g, B, H, T, 64, dtype=dtype)
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(B, T, T).contiguous()
+    return qkv, dO, mask
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,T", [(1, 1, 64), (2, 3, 128), (1, 2, 192), (2, 2, 256), (1, 12, 512)])
+@pytest.mark.parametrize("train", [False, True])
+def test_attn_fwd_bwd_causal(mt, dtype, B, H, T, train):
+    qkv, dO, mask = make(B, H, T, dtype, seed=T + B)
+    seed = 4242
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), train, seed)
+    want_o = ops.scaled_dot_prod_attn_fwd(f64(qkv), mask, train, seed)
+    close(o, want_o, dtype, "O")
+    ms, ls = ops.scaled_dot_prod_attn_stats(f64(qkv), mask)
+    assert acts[2] is o and acts[0].shape == (B, H, T)
+    close(acts[0], ms, torch.float32 if dtype == torch.float32 else dtype, "ms")
+    close(acts[1], ls, torch.float32 if dtype == torch.float32 else dtype, "ls")
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    wq, wk, wv = ops.scaled_dot_prod_attn_bkwd(f64(dO), f64(qkv), mask, train, seed)
+    close(dq, wq, dtype, "dq")
+    close(dk, wk, dtype, "dk")
+    close(dv, wv, dtype, "dv")
+    # deterministic (no atomics)
+    dq2, dk2, dv2 = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_config2_shape(mt, dtype):
+    # BASELINE config 2: B=8, H=12, T=1024, dh=64 (oracle on a 2-batch slice to bound CPU time)
+    B, H, T = 8, 12, 1024
+    qkv, dO, mask = make(B, H, T, dtype, seed=2)
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), False)
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), False)
+    sl = slice(6, 8)
+    want_o = ops.scaled_dot_prod_attn_fwd(f64(qkv[sl]), mask[sl], False)
+    close(o[sl], want_o, dtype, "O")
+    wq, wk, wv = ops.scaled_dot_prod_attn_bkwd(f64(dO[sl]), f64(qkv[sl]), mask[sl], False)
+    close(dq[sl], wq, dtype, "dq")
+    close(dk[sl], wk, dtype, "dk")
+    close(dv[sl], wv, dtype, "dv")
+    # size-independent property at full size: T=1 prefix -> first output row equals 0.9 * v[0]
+    assert torch.allclose(o[:, :, 0].float().cpu(), 0.9 * qkv[:, :, 2, 0].float(), rtol=2e-2, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("train", [False, True])
+def test_attn_padding_mask(mt, dtype, train):
+    # tril AND key-padding AND packing (block-diagonal) -- sub-masks of the causal mask, as the
+    # training collator builds them; every row keeps its diagonal.
+    B, H, T = 2, 2, 256
+    qkv, dO, mask = make(B, H, T, dtype, seed=9)
+    mask = mask.clone()
+    mask[0, :, 100:130] = False                      # padded keys ...
+    mask[0, 200:, :200] = False                      # second packed sequence cannot see the first
+    mask[1, 64:, :64] = False
+    idx = torch.arange(T)
+    mask[:, idx, idx] = True                         # ... but a token always sees itself
+    seed = 77
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), train, seed)
+    close(o, ops.scaled_dot_prod_attn_fwd(f64(qkv), mask, train, seed), dtype, "O")
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    wq, wk, wv = ops.scaled_dot_prod_attn_bkwd(f64(dO), f64(qkv), mask, train, seed)
+    close(dq, wq, dtype, "dq")
+    close(dk, wk, dtype, "dk")
+    close(dv, wv, dtype, "dv")
+
+
+def test_attn_dropout_mask_bits(mt):
+    # P with q = 0, k = 0 is uniform over visible keys; with v = one-hot(key % 64) the train-mode
+    # output row i, column c is (#kept keys j<=i with j%64==c)/(i+1): recovers the keep mask exactly.
+    B, H, T = 1, 2, 128
+    qkv = torch.zeros(B, H, 3, T, 64)
+    qkv[:, :, 2, torch.arange(T), torch.arange(T) % 64] = 1.0
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(B, T, T).contiguous()
+    seed = 31337
+    o, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), True, seed)
+    keep = ops.attn_keep(B, H, T, seed).to(torch.float64)
+    want = torch.einsum("bhqk,kc->bhqc", keep * mask.unsqueeze(1), torch.eye(64, dtype=torch.float64).repeat(2, 1))
+    want = want / torch.arange(1, T + 1, dtype=torch.float64).view(1, 1, T, 1)
+    assert torch.allclose(f64(o), want, rtol=1e-5, atol=1e-7)
+
+
+def test_attn_strided_views_fused_qkv_layout(mt):
+    # q/k/v as column slices of one [B*T, H*3*dh] buffer, O written into [B,T,H*dh]
+    B, H, T = 2, 4, 128
+    g = gen(21)
+    buf = randn(g, B * T, H * 3 * 64, dtype=torch.bfloat16).to(DEV)
+    v5 = buf.view(B, T, H, 3, 64)
+    q, k, v = (v5[:, :, :, c].permute(0, 2, 1, 3) for c in range(3))
+    out = torch.empty(B, T, H * 64, dtype=torch.bfloat16, device=DEV)
+    o, ms, ls = mt.attn_fwd_t(q, k, v, None, False, 0, out=out.view(B, T, H, 64).permute(0, 2, 1, 3))
+    qkv = torch.stack((q, k, v), dim=2).contiguous()
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=DEV)).expand(B, T, T)
+    o_ref, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qkv, mask, False)
+    assert torch.equal(o, o_ref)
+    assert torch.equal(out.view(B, T, H, 64).permute(0, 2, 1, 3), o_ref)
+
+
+def test_attn_rejects_bad_shapes(mt):
+    _lib = __import__("importlib").import_module("pre-tjax_amd._lib")
+    qkv = torch.zeros(1, 1, 3, 96, 64, device=DEV)
+    with pytest.raises(AssertionError):
+        mt.t_scaled_dot_prod_attn_fwd3_t(qkv, None, False)
+    q = torch.zeros(1, 1, 64, 32, device=DEV)
+    with pytest.raises(_lib.PtjError):
+        mt.attn_fwd_t(q, q, q, None, False, 0)
