@@ -55,12 +55,21 @@ int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* 
  * t_layernorm_bkwd2_p_k/_t (model_triton.py:1664-1726) with a deterministic
  * two-stage reduction instead of float atomics.  `workspace` must hold
  * ptj_layernorm_bwd_workspace_bytes(rows, cols) bytes when dgamma != NULL
- * (may be NULL otherwise).  gamma may be NULL when dx == NULL. */
+ * (may be NULL otherwise).  gamma may be NULL when dx == NULL.  `residual` (nullable,
+ * contiguous [rows, cols]) is added to dx: the `blck_dloss_dx + dloss_dx` of the block
+ * backward (model_triton.py:2036, 2190) without a separate pass. */
 size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols);
-int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma,
+int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const void* residual,
                       void* dx, void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes,
                       int64_t rows, int64_t cols, int64_t dy_row_stride, int64_t x_row_stride,
                       int64_t dx_row_stride, int dtype, void* stream);
+
+/* Column sums out[c] = sum_r x[r, c] (bias gradients: the `.sum(dim=0)` of
+ * t_linear_bkwd2_p, model_triton.py:426).  Two-stage, fixed order.  `workspace`:
+ * ptj_colsum_workspace_bytes(rows, cols) bytes. */
+size_t ptj_colsum_workspace_bytes(int64_t rows, int64_t cols);
+int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes,
+               int64_t rows, int64_t cols, int64_t x_row_stride, int dtype, void* stream);
 
 /* tanh-GELU forward / backward on a flat array of n elements.
  * Replace t_gelu_fwd_k/_t (model_triton.py:237-260) and t_gelu_bkwd2_k/_t (:274-304). */
@@ -97,11 +106,13 @@ int ptj_log_softmax_bwd(const void* dy, const void* x, void* dx, int64_t rows, i
  *   loss    float [1]  (fp32 regardless of dtype) = -mean_{label!=0} log_softmax(x)[label];
  *   count   int64 [1]  = number of labels != 0;
  *   dlogits = (softmax(x) - onehot(label))/count on rows with label != 0, else 0.
+ *   pred    int64 [rows] or NULL: argmax of each logits row (lowest index on ties), the
+ *           input of the reference's accuracy() (loss_and_optimizer_triton.py:199-200);
  * dlogits may alias logits (in-place).  `workspace`: ptj_ce_workspace_bytes(rows) bytes.
  * Deterministic (no atomics).  count == 0 gives loss = NaN as the reference does. */
 size_t ptj_ce_workspace_bytes(int64_t rows);
 int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64_t* count,
-                   void* dlogits, void* workspace, size_t workspace_bytes,
+                   void* dlogits, int64_t* pred, void* workspace, size_t workspace_bytes,
                    int64_t rows, int64_t cols, int64_t logits_row_stride, int64_t dlogits_row_stride,
                    int dtype, void* stream);
 

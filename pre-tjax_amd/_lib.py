@@ -23,7 +23,9 @@ SIGNATURES = {
     "ptj_last_error": (_c.c_char_p, []),
     "ptj_layernorm_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
-    "ptj_layernorm_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64, _int, _p]),
+    "ptj_layernorm_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64, _int, _p]),
+    "ptj_colsum_workspace_bytes": (_sz, [_i64, _i64]),
+    "ptj_colsum": (_int, [_p, _p, _p, _sz, _i64, _i64, _i64, _int, _p]),
     "ptj_gelu_fwd": (_int, [_p, _p, _i64, _int, _p]),
     "ptj_gelu_bwd": (_int, [_p, _p, _p, _i64, _int, _p]),
     "ptj_dropout": (_int, [_p, _p, _i64, _i64, _i64, _i64, _int, _i64, _int, _p]),
@@ -31,7 +33,7 @@ SIGNATURES = {
     "ptj_log_softmax_fwd": (_int, [_p, _p, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_log_softmax_bwd": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_ce_workspace_bytes": (_sz, [_i64]),
-    "ptj_ce_fwd_bwd": (_int, [_p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
+    "ptj_ce_fwd_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "ptj_gemm": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p, _sz, _int, _p]),
     "ptj_attn_workspace_bytes": (_sz, [_i64, _i64, _i64]),

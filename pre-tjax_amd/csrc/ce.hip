@@ -31,10 +31,12 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restric
 template <typename T, int ITERS, bool CACHED>
 __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict__ labels, const T* logits,
                                                        T* dlogits, float* __restrict__ row_loss,
+                                                       int64_t* __restrict__ pred,
                                                        const int64_t* __restrict__ count, int64_t rows, int cols,
                                                        int64_t xs, int64_t dxs) {
     constexpr int VEC = VecOf<T>::N;
     __shared__ float smem[16];
+    __shared__ int smin[16];
     __shared__ float s_xy;
     const int t = threadIdx.x;
     const float inv_cnt = 1.0f / (float)(*count);
@@ -79,6 +81,41 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
             }
         }
         m = row_reduce<CE_THREADS, true>(m, smem);
+        if (pred != nullptr) {
+            // argmax = lowest column whose logit equals the row maximum
+            int best = 0x7fffffff;
+            if constexpr (CACHED) {
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const int e = (t + it * CE_THREADS) * VEC + j - mis;
+                        if (v[it][j] == m && e < best) best = e;
+                    }
+            } else {
+                for (int vi = t; vi < nvec; vi += CE_THREADS) {
+                    float w[VEC];
+                    load_vec<T, VEC>(xb + (int64_t)vi * VEC, w);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const int e = vi * VEC + j - mis;
+                        if (e >= 0 && e < cols && w[j] == m && e < best) best = e;
+                    }
+                }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const int other = __shfl_xor(best, o, 64);
+                best = other < best ? other : best;
+            }
+            if ((t & 63) == 0) smin[t >> 6] = best;
+            __syncthreads();
+            if (t == 0) {
+                int b = smin[0];
+                for (int i = 1; i < CE_THREADS / 64; ++i) b = smin[i] < b ? smin[i] : b;
+                pred[row] = b;
+            }
+        }
         float s = 0.f;
         if constexpr (CACHED) {
 #pragma unroll
@@ -169,8 +206,8 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(const float* __restri
 }
 
 template <typename T>
-int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits, void* ws,
-            int64_t rows, int64_t cols, int64_t xs, int64_t dxs, hipStream_t st) {
+int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits, int64_t* pred,
+            void* ws, int64_t rows, int64_t cols, int64_t xs, int64_t dxs, hipStream_t st) {
     constexpr int VEC = VecOf<T>::N;
     constexpr int ITERS = 64 / VEC;  // 64 cached floats per thread
     float* row_loss = (float*)ws;
@@ -180,10 +217,10 @@ int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* cou
     const bool cached = (cols + VEC) <= (int64_t)CE_THREADS * ITERS * VEC;
     if (cached)
         hipLaunchKernelGGL((ce_row_kernel<T, ITERS, true>), dim3(grid), dim3(1024), 0, st, labels, (const T*)logits,
-                           (T*)dlogits, row_loss, (const int64_t*)count, rows, (int)cols, xs, dxs);
+                           (T*)dlogits, row_loss, pred, (const int64_t*)count, rows, (int)cols, xs, dxs);
     else
         hipLaunchKernelGGL((ce_row_kernel<T, 1, false>), dim3(grid), dim3(1024), 0, st, labels, (const T*)logits,
-                           (T*)dlogits, row_loss, (const int64_t*)count, rows, (int)cols, xs, dxs);
+                           (T*)dlogits, row_loss, pred, (const int64_t*)count, rows, (int)cols, xs, dxs);
     PTJ_CHECK_LAUNCH();
     hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)row_loss, rows,
                        (const int64_t*)count, loss);
@@ -198,7 +235,7 @@ extern "C" {
 size_t ptj_ce_workspace_bytes(int64_t rows) { return rows > 0 ? (size_t)rows * sizeof(float) : 0; }
 
 int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
-                   void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t xs, int64_t dxs,
+                   int64_t* pred, void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t xs, int64_t dxs,
                    int dtype, void* stream) {
     PTJ_CHECK_ARG(labels && logits && loss && count && dlogits, "ce_fwd_bwd: null pointer");
     PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 30), "ce_fwd_bwd: bad shape %lld x %lld", (long long)rows,
@@ -214,8 +251,8 @@ int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64
                   "ce_fwd_bwd: logits and dlogits rows must have equal 16-byte misalignment");
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case PTJ_F32: return ce_impl<float>(labels, logits, loss, count, dlogits, workspace, rows, cols, xs, dxs, st);
-        case PTJ_BF16: return ce_impl<bf16>(labels, logits, loss, count, dlogits, workspace, rows, cols, xs, dxs, st);
+        case PTJ_F32: return ce_impl<float>(labels, logits, loss, count, dlogits, pred, workspace, rows, cols, xs, dxs, st);
+        case PTJ_BF16: return ce_impl<bf16>(labels, logits, loss, count, dlogits, pred, workspace, rows, cols, xs, dxs, st);
         default: return ptj_set_error(PTJ_ERR_INVALID, "ce_fwd_bwd: unknown dtype %d", dtype);
     }
 }

@@ -100,8 +100,8 @@ constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave ho
 
 template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
 __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
-    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, T* __restrict__ dx,
-    float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs) {
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
+    T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs) {
     __shared__ float smem[16];
     constexpr int RPB = LnBwdGeom<TPR>::ROWS_PER_BLOCK;
     const int t = threadIdx.x % TPR;
@@ -169,6 +169,15 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
             for (int it = 0; it < ITERS; ++it)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) d.v[it][j] = (d.v[it][j] - mg - r.v[it][j] * mgx) * rstd;
+            if (res != nullptr) {
+                // residual branch: the sum is formed from the storage-rounded LayerNorm gradient,
+                // as two separate passes would
+                r.load(res + row * (int64_t)cols, nvec, t, 0.f);
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) d.v[it][j] = r.v[it][j] + to_f32(from_f32<T>(d.v[it][j]));
+            }
             d.store(dx + row * dxs, nvec, t);
         }
     }
@@ -377,6 +386,83 @@ __global__ __launch_bounds__(256) void dropout_kernel(const T* __restrict__ x, c
 }
 
 // ---------------------------------------------------------------------------------
+// Column sums, two stages.  Stage 1: block (bx, by) sums rows [by*rps, (by+1)*rps) of the
+// 128*VEC columns starting at bx*128*VEC into part[by][col].  Stage 2 reuses the
+// LayerNorm partial reducer layout (part[p][1][cols] with a single "which").
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(128) void colsum_stage1_kernel(const T* __restrict__ x, float* __restrict__ part,
+                                                            int64_t rows, int cols, int64_t xs, int rows_per_split) {
+    const int c0 = (blockIdx.x * 128 + threadIdx.x) * VEC;
+    if (c0 >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+    const int64_t r1 = r0 + rows_per_split < rows ? r0 + rows_per_split : rows;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int64_t r = r0; r < r1; ++r) {
+        float v[VEC];
+        load_vec<T, VEC>(x + r * xs + c0, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += v[j];
+    }
+    float* dst = part + (int64_t)blockIdx.y * cols + c0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) dst[j] = acc[j];
+}
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_stage2_kernel(const float* __restrict__ part, int nparts, int cols,
+                                                            T* __restrict__ out) {
+    __shared__ float sm[8][33];
+    const int cx = threadIdx.x & 31, py = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + cx;
+    float s = 0.f;
+    if (c < cols)
+        for (int p = py; p < nparts; p += 8) s += part[(int64_t)p * cols + c];
+    sm[py][cx] = s;
+    __syncthreads();
+    if (py == 0 && c < cols) {
+        float r = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r += sm[i][cx];
+        out[c] = from_f32<T>(r);
+    }
+}
+
+inline void colsum_geometry(int64_t rows, int64_t cols, int vec, int* gx, int* splits, int* rps) {
+    *gx = (int)((cols + 128 * vec - 1) / (128 * vec));
+    int64_t s = 2048 / *gx;
+    if (s < 1) s = 1;
+    if (s > (rows + 31) / 32) s = (rows + 31) / 32;
+    if (s < 1) s = 1;
+    *rps = (int)((rows + s - 1) / s);
+    *splits = (int)((rows + *rps - 1) / *rps);
+}
+
+template <typename T>
+int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t rows, int64_t cols, int64_t xs,
+                hipStream_t st) {
+    constexpr int FV = VecOf<T>::N;
+    const bool vok = (cols % FV == 0) && (xs % FV == 0) && ptj_aligned16(x);
+    const int vec = vok ? FV : 1;
+    int gx, splits, rps;
+    colsum_geometry(rows, cols, vec, &gx, &splits, &rps);
+    const size_t need = (size_t)splits * cols * sizeof(float);
+    if (!ws || ws_bytes < need) return ptj_set_error(PTJ_ERR_WORKSPACE, "colsum: workspace %zu < %zu bytes", ws_bytes, need);
+    if (vok)
+        hipLaunchKernelGGL((colsum_stage1_kernel<T, FV>), dim3(gx, splits), dim3(128), 0, st, (const T*)x, (float*)ws,
+                           rows, (int)cols, xs, rps);
+    else
+        hipLaunchKernelGGL((colsum_stage1_kernel<T, 1>), dim3(gx, splits), dim3(128), 0, st, (const T*)x, (float*)ws,
+                           rows, (int)cols, xs, rps);
+    PTJ_CHECK_LAUNCH();
+    hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(256), 0, st,
+                       (const float*)ws, splits, (int)cols, (T*)out);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+// ---------------------------------------------------------------------------------
 // Dispatch helpers
 // ---------------------------------------------------------------------------------
 struct RowCfg {
@@ -456,11 +542,12 @@ inline int ln_bwd_grid(int64_t rows, int tpr) {
 }
 
 template <typename T>
-int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
+int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const void* res, void* dx, void* dgamma,
+                       void* dbeta,
                        void* ws, size_t ws_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs, int64_t dxs,
                        hipStream_t st) {
     RowCfg cfg;
-    const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx}, {dys, xs, dx ? dxs : 0});
+    const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx, res}, {dys, xs, dx ? dxs : 0});
     if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
         return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: cols=%lld too large", (long long)cols);
     const int grid = ln_bwd_grid(rows, cfg.tpr);
@@ -473,7 +560,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, void* d
     }
 #define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_)                                                                   \
     hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
-                       dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (T_*)dx, \
+                       dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (const T_*)res, (T_*)dx, \
                        (float*)ws, rows, (int)cols, dys, xs, dxs)
 #define LAUNCH(T_, V_, TPR_, IT_)                                     \
     do {                                                              \
@@ -607,21 +694,46 @@ size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
     return (size_t)512 * 2 * (size_t)cols * sizeof(float);
 }
 
-int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
+int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const void* residual, void* dx, void* dgamma,
+                      void* dbeta,
                       void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
                       int64_t dxs, int dtype, void* stream) {
     PTJ_CHECK_ARG(dy && x, "layernorm_bwd: null dy/x");
     PTJ_CHECK_ARG(dx || dgamma, "layernorm_bwd: nothing to compute (dx and dgamma both null)");
     PTJ_CHECK_ARG(!dx || gamma, "layernorm_bwd: dx requested without gamma");
+    PTJ_CHECK_ARG(!residual || dx, "layernorm_bwd: residual given without dx");
     PTJ_CHECK_ARG((dgamma == nullptr) == (dbeta == nullptr), "layernorm_bwd: dgamma and dbeta must be given together");
     PTJ_CHECK_ARG(rows >= 1 && cols >= 2, "layernorm_bwd: need rows >= 1 and cols >= 2");
     PTJ_CHECK_ARG(dys >= cols && xs >= cols && (!dx || dxs >= cols), "layernorm_bwd: row stride smaller than cols");
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype,
-                 (layernorm_bwd_impl<float>(dy, x, gamma, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols,
+                 (layernorm_bwd_impl<float>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols,
                                             dys, xs, dxs, st)),
-                 (layernorm_bwd_impl<bf16>(dy, x, gamma, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols, dys,
+                 (layernorm_bwd_impl<bf16>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols, dys,
                                            xs, dxs, st)));
+}
+
+size_t ptj_colsum_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    int gx, splits, rps;
+    colsum_geometry(rows, cols, 1, &gx, &splits, &rps);   // scalar geometry bounds the vector one
+    int gx2, splits2, rps2;
+    colsum_geometry(rows, cols, 8, &gx2, &splits2, &rps2);
+    int gx3, splits3, rps3;
+    colsum_geometry(rows, cols, 4, &gx3, &splits3, &rps3);
+    int m = splits > splits2 ? splits : splits2;
+    m = m > splits3 ? m : splits3;
+    return (size_t)m * cols * sizeof(float);
+}
+
+int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols,
+               int64_t xs, int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 31), "colsum: bad shape");
+    PTJ_CHECK_ARG(x && out, "colsum: null pointer");
+    PTJ_CHECK_ARG(xs >= cols, "colsum: row stride smaller than cols");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (colsum_impl<float>(x, out, workspace, workspace_bytes, rows, cols, xs, st)),
+                 (colsum_impl<bf16>(x, out, workspace, workspace_bytes, rows, cols, xs, st)));
 }
 
 int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream) {

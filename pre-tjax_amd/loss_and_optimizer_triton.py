@@ -6,25 +6,97 @@ from ._lib import check, dtype_code, lib, ptr, require_gpu, stream
 from .model_triton import _workspace
 
 
-def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Tensor, inplace=False):
+def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Tensor, inplace=False, want_pred=False):
     """Fused log-softmax + mean cross-entropy forward and backward
     (reference: loss_and_optimizer_triton.py:176-197).
 
     Returns ``(loss[1] fp32, nonzero_count 0-d int64, dloss_dlogits like x_logits)``.
     With ``inplace=True`` the gradient overwrites ``x_logits`` (an extension: the
-    reference always allocates)."""
+    reference always allocates).  With ``want_pred=True`` a fourth value is returned:
+    the row-wise argmax of the logits (int64, shaped like ``y_labels``), computed in
+    the same pass -- the input of ``accuracy``."""
     require_gpu(y_labels, x_logits)
     shape = x_logits.shape
     labels = y_labels.reshape(-1).to(torch.int64).contiguous()
-    x2 = x_logits.reshape(labels.numel(), -1)
-    if not x2.is_contiguous():
+    x2 = x_logits.reshape(labels.numel(), -1)     # a view for row-padded logits buffers
+    if x2.stride(1) != 1:
         x2 = x2.contiguous()
     rows, cols = x2.shape
     loss = torch.empty(1, dtype=torch.float32, device=x2.device)
     count = torch.empty((), dtype=torch.int64, device=x2.device)
-    dx = x2 if inplace else torch.empty_like(x2)
+    if inplace:
+        dx = x2
+    else:  # same row pitch as the logits, so rows keep their 16-byte phase
+        dx = torch.empty_strided((rows, cols), (x2.stride(0), 1), dtype=x2.dtype, device=x2.device)
+    pred = torch.empty(rows, dtype=torch.int64, device=x2.device) if want_pred else None
     ws_bytes = lib().ptj_ce_workspace_bytes(rows)
     ws = _workspace(ws_bytes, x2.device, "ce")
-    check(lib().ptj_ce_fwd_bwd(ptr(labels), ptr(x2), ptr(loss), ptr(count), ptr(dx), ptr(ws), ws_bytes, rows, cols,
+    check(lib().ptj_ce_fwd_bwd(ptr(labels), ptr(x2), ptr(loss), ptr(count), ptr(dx), ptr(pred), ptr(ws), ws_bytes, rows, cols,
                                x2.stride(0), dx.stride(0), dtype_code(x2), stream()), "ptj_ce_fwd_bwd")
-    return loss, count, dx.reshape(shape)
+    dx = dx.view(shape) if inplace else dx.reshape(shape)
+    if want_pred:
+        return loss, count, dx, pred.reshape(y_labels.shape)
+    return loss, count, dx
+
+
+def accuracy_from_pred(y_labels, pred):
+    """loss_and_optimizer_triton.py:199-200 given the row-wise argmax."""
+    hit = (y_labels == pred).to(torch.float32)
+    return torch.nanmean(torch.where(y_labels != 0, hit, torch.full_like(hit, float("nan"))))
+
+
+def t_loss_bkwd3_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
+    """One forward+backward (reference: loss_and_optimizer_triton.py:279-289).
+    y int [B,T+1] -> (grads nest, (loss, acc, non-pad fraction))."""
+    from .model_triton import t_gpt2_bkwd3_p_t, t_gpt2_forward_with_acts_t
+    y_in = y[:, :-1]
+    y_out = y[:, 1:]
+    logits, acts = t_gpt2_forward_with_acts_t(params, y_in, y_mask, y_indices, train, p_gen_aux)
+    loss_val, tokens_count, dloss_dx, pred = t_avg_cross_entropy_loss_bkwd3_t(y_out, logits, inplace=True,
+                                                                             want_pred=True)
+    grads = t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y_in, y_mask, y_indices, train, p_gen_aux)
+    acc = accuracy_from_pred(y_out, pred)
+    return grads, (loss_val, acc, tokens_count / y_out.numel())
+
+
+def sample_p_gen_aux(params, generator=None):
+    """1 + 3L dropout seeds in [0, 1e6) (loss_and_optimizer_triton.py:318-325) drawn on
+    the host: no device round trips."""
+    n = 1 + 3 * (len(params) - 3)
+    return torch.randint(0, 1_000_000, (n,), generator=generator).tolist()
+
+
+def init_adam_w(params):
+    """fp32 first/second moments shaped like `params` (reference :362-363)."""
+    return [[[torch.zeros_like(p, dtype=torch.float32) for p in grp] for grp in params] for _ in range(2)]
+
+
+def adam_w_in_place(master, grads, lr, betas, epsilon, moments, i, weight_decay=0.0, weight_decay_mask=None,
+                    shadow=None):
+    """AdamW of the reference (:376-401: t = i+1, bias-corrected moments, decay scaled by
+    lr) on fp32 master weights, with torch's multi-tensor ops instead of per-tensor Python
+    loops.  `shadow` (optional nest of low-precision copies) is refreshed from the masters."""
+    t = i + 1
+    flat_p = [p for grp in master for p in grp]
+    flat_g = [g.to(torch.float32) for grp in grads for g in grp]
+    flat_m = [m for grp in moments[0] for m in grp]
+    flat_v = [v for grp in moments[1] for v in grp]
+    b1, b2 = betas
+    torch._foreach_mul_(flat_m, b1)
+    torch._foreach_add_(flat_m, flat_g, alpha=1 - b1)
+    torch._foreach_mul_(flat_v, b2)
+    torch._foreach_addcmul_(flat_v, flat_g, flat_g, value=1 - b2)
+    denom = torch._foreach_div(flat_v, 1 - b2 ** t)
+    torch._foreach_sqrt_(denom)
+    torch._foreach_add_(denom, epsilon)
+    if weight_decay:
+        flags = [True if weight_decay_mask is None else bool(weight_decay_mask[gi][pi])
+                 for gi, grp in enumerate(master) for pi, _ in enumerate(grp)]
+        decayed = [p for p, f in zip(flat_p, flags) if f]
+        if decayed:
+            torch._foreach_mul_(decayed, 1 - lr * weight_decay)
+    torch._foreach_addcdiv_(flat_p, flat_m, denom, value=-lr / (1 - b1 ** t))
+    if shadow is not None:
+        flat_s = [s for grp in shadow for s in grp]
+        torch._foreach_copy_(flat_s, flat_p)
+    return master, moments

@@ -138,7 +138,7 @@ def t_layernorm_fwd_t(layer_params, x: torch.Tensor):
     return out.reshape(x.shape)
 
 
-def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p):
+def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None):
     require_gpu(dloss_dx, x)
     d2, x2 = _rows2d(dloss_dx), _rows2d(x)
     assert d2.shape == x2.shape and d2.dtype == x2.dtype
@@ -151,7 +151,10 @@ def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p):
     if want_p:
         ws_bytes = lib().ptj_layernorm_bwd_workspace_bytes(rows, cols)
         ws = _workspace(ws_bytes, x2.device, "ln_bwd")
-    check(lib().ptj_layernorm_bwd(ptr(d2), ptr(x2), ptr(gamma), ptr(dx), ptr(dg), ptr(db), ptr(ws), ws_bytes,
+    if residual is not None:
+        assert want_dx and residual.shape == x.shape and residual.dtype == x2.dtype
+        residual = residual.contiguous()
+    check(lib().ptj_layernorm_bwd(ptr(d2), ptr(x2), ptr(gamma), ptr(residual), ptr(dx), ptr(dg), ptr(db), ptr(ws), ws_bytes,
                                   rows, cols, d2.stride(0), x2.stride(0), dx.stride(0) if want_dx else 0,
                                   dtype_code(x2), stream()), "ptj_layernorm_bwd")
     return (dx.reshape(dloss_dx.shape) if want_dx else None), dg, db
@@ -167,11 +170,25 @@ def t_layernorm_bkwd2_x_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor)
     return dx
 
 
-def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor):
-    """dx, (dgamma, dbeta) from one read of dy and x (fusion of the two reference
-    launches at model_triton.py:2033-2034)."""
-    dx, dg, db = _layernorm_bwd(dloss_dx, layer_params, x, True, True)
+def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, residual=None):
+    """dx (+ residual), (dgamma, dbeta) from one read of dy and x (fusion of the two
+    reference launches at model_triton.py:2033-2034 and of the residual add at :2036)."""
+    dx, dg, db = _layernorm_bwd(dloss_dx, layer_params, x, True, True, residual)
     return dx, (dg, db)
+
+
+def colsum_t(x: torch.Tensor):
+    """Sum over all leading dimensions: the bias gradient `.sum(dim=0)` of the reference's
+    t_linear_bkwd2_p (model_triton.py:426), deterministic."""
+    require_gpu(x)
+    x2 = _rows2d(x)
+    rows, cols = x2.shape
+    out = torch.empty(cols, dtype=x2.dtype, device=x2.device)
+    ws_bytes = lib().ptj_colsum_workspace_bytes(rows, cols)
+    ws = _workspace(ws_bytes, x2.device, "colsum")
+    check(lib().ptj_colsum(ptr(x2), ptr(out), ptr(ws), ws_bytes, rows, cols, x2.stride(0), dtype_code(x2), stream()),
+          "ptj_colsum")
+    return out
 
 
 # ----------------------------------------------------------------------------------
@@ -329,3 +346,164 @@ def t_scaled_dot_prod_attn_bkwd3_t(dloss_dx, acts, qkv: torch.Tensor, mask: torc
     q, k, v = (_aligned_view(t) for t in torch.unbind(qkv, dim=2))
     ms, ls, o = acts
     return attn_bwd_t(_aligned_view(dloss_dx), q, k, v, _aligned_view(o), ms, ls, mask, train, p_gen_aux)
+
+
+# ----------------------------------------------------------------------------------
+# GPT-2 composites  (reference: model_triton.py:2334-2351 t_gpt2_tlayers_fwd3_t,
+# :2535-2539 t_gpt2_forward_with_acts_t, :2489-2521 / :2583-2593 backward)
+#
+# Same call order and arithmetic as the reference's fwd3_t / bkwd3_t chain, with the
+# host-side "linking" restated for the hardware:
+#   * Q, K and V of all heads come from ONE [N,D]x[D,3D] product (the reference stacks
+#     the LayerNorm output three times and runs a broadcast matmul, :1051-1053); the
+#     attention kernels read/write strided slices of that buffer and of the [N,D]
+#     head-merged output, so no head transposes or stack/sum copies exist;
+#   * residual + dropout, and LayerNorm dx + dgamma/dbeta + residual, are single passes;
+#   * the FFN pre-activation is saved instead of recomputed (:1415-1418 recomputes it);
+#   * the LM-head logits live in a row-padded buffer (pitch = V rounded up to 64) so
+#     that every row is 16-byte aligned; the loss gradient overwrites it in place.
+# ----------------------------------------------------------------------------------
+VOCAB_PAD = 64
+
+
+def _padded_logits(n_rows, vocab, dtype, device):
+    pitch = (vocab + VOCAB_PAD - 1) // VOCAB_PAD * VOCAB_PAD
+    buf = torch.empty((n_rows, pitch), dtype=dtype, device=device)
+    return buf[:, :vocab]
+
+
+def t_embed_fwd(layer_params, x):
+    """model_triton.py:166-167 (torch gather, as in the reference)."""
+    return layer_params[0][x] * math.sqrt(layer_params[0].shape[1])
+
+
+def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
+    """One block (model_triton.py:2214-2223).  y [B,T,D] -> (y_out, acts)."""
+    if not train:
+        p_gen_aux = [0, 0, 0]
+    ln1g, ln1b, wqkv, wo, ln2g, ln2b, w1, b1, w2, b2 = layer_params
+    B, T, D = y.shape
+    H, _, dh, _ = wqkv.shape
+    N = B * T
+    x_in = y.reshape(N, D)
+    h1 = t_layernorm_fwd_t((ln1g, ln1b), x_in)
+    qkv = matmul_t(h1, wqkv.view(H * 3 * dh, D).t())                     # [N, H*3*dh]
+    v5 = qkv.view(B, T, H, 3, dh)
+    q, k, v = (v5[:, :, :, c].permute(0, 2, 1, 3) for c in range(3))     # [B,H,T,dh] views
+    o2 = torch.empty((N, D), dtype=y.dtype, device=y.device)
+    o4 = o2.view(B, T, H, dh).permute(0, 2, 1, 3)
+    _, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux[0], out=o4)
+    a_out = matmul_t(o2, wo.t())
+    x_mid = dropout_add_t(a_out, x_in, train, p_gen_aux[1])
+    h2 = t_layernorm_fwd_t((ln2g, ln2b), x_mid)
+    f1 = matmul_t(h2, w1.t(), b1)
+    g1 = t_gelu_fwd_t(f1)
+    f2 = matmul_t(g1, w2.t(), b2)
+    x_out = dropout_add_t(f2, x_mid, train, p_gen_aux[2])
+    acts = (x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1)
+    return x_out.view(B, T, D), acts
+
+
+def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_aux=None):
+    """Backward of one block (model_triton.py:2291-2299 and the sub-block VJPs :2021-2039,
+    :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order)."""
+    if not train:
+        p_gen_aux = [0, 0, 0]
+    ln1g, ln1b, wqkv, wo, ln2g, ln2b, w1, b1, w2, b2 = layer_params
+    x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1 = acts
+    H, _, dh, D = wqkv.shape
+    N = x_in.shape[0]
+    T = ms.shape[2]
+    B = N // T
+    # ---- sub-block 2: x_out = x_mid + dropout(ffn(ln2(x_mid)))
+    d = t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2])
+    db2 = colsum_t(d)
+    dw2 = matmul_t(d.t(), g1)                                           # [D,F]
+    dg1 = matmul_t(d, w2)                                               # [N,F]
+    df1 = t_gelu_bkwd2_t(dg1, f1)
+    db1 = colsum_t(df1)
+    dw1 = matmul_t(df1.t(), h2)                                         # [F,D]
+    dh2 = matmul_t(df1, w1)                                             # [N,D]
+    dx_mid, (dln2g, dln2b) = layernorm_bkwd2_t(dh2, (ln2g, ln2b), x_mid, residual=dloss_dx)
+    # ---- sub-block 1: x_mid = x_in + dropout(attn(ln1(x_in)))
+    d = t_dropout_bkwd2_t(dx_mid, None, train, p_gen_aux[1])
+    dwo = matmul_t(d.t(), o2)                                           # [D,D]
+    do2 = matmul_t(d, wo)                                               # [N,D] = [B,T,H,dh]
+    v5 = qkv.view(B, T, H, 3, dh)
+    q, k, v = (v5[:, :, :, c].permute(0, 2, 1, 3) for c in range(3))
+    dqkv = torch.empty_like(qkv)
+    d5 = dqkv.view(B, T, H, 3, dh)
+    outs = tuple(d5[:, :, :, c].permute(0, 2, 1, 3) for c in range(3))
+    o4 = o2.view(B, T, H, dh).permute(0, 2, 1, 3)
+    do4 = do2.view(B, T, H, dh).permute(0, 2, 1, 3)
+    attn_bwd_t(do4, q, k, v, o4, ms, ls, mask, train, p_gen_aux[0], out=outs)
+    dwqkv = matmul_t(dqkv.t(), h1).view(H, 3, dh, D)                    # [H*3*dh, D]
+    dh1 = matmul_t(dqkv, wqkv.view(H * 3 * dh, D))                      # [N,D]
+    dx_in, (dln1g, dln1b) = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid)
+    return dx_in, [dln1g, dln1b, dwqkv, dwo, dln2g, dln2b, dw1, db1, dw2, db2]
+
+
+def t_gpt2_tlayers_fwd3_t(params, y, mask, indices, train=True, p_gen_aux=None):
+    """model_triton.py:2334-2351.  y int [B,T] -> (h [B,T,D], acts)."""
+    L = len(params) - 3
+    if not train:
+        p_gen_aux = [0] * (1 + 3 * L)
+    T = y.shape[1]
+    assert T <= params[1][0].shape[0], "sequence longer than the positional table"
+    x = t_embed_fwd(params[0], y) + params[1][0][:T]
+    x = t_dropout_fwd_t(x, train, p_gen_aux[0])
+    layer_acts = []
+    for i, lp in enumerate(params[2:-1]):
+        x, a = t_gpt2_tlayer_fwd3_t(lp, x, mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i])
+        layer_acts.append(a)
+    h = t_layernorm_fwd_t(params[-1], x)
+    return h, [layer_acts, x]
+
+
+def t_gpt2_forward_with_acts_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
+    """model_triton.py:2535-2539: -> (logits [B,T,V], acts).  The logits are a view of a
+    row-padded buffer (unit column stride)."""
+    h, acts = t_gpt2_tlayers_fwd3_t(params, y, y_mask, y_indices, train, p_gen_aux)
+    B, T, D = h.shape
+    wemb, bemb = params[0]
+    V = wemb.shape[0]
+    logits = _padded_logits(B * T, V, h.dtype, h.device)
+    matmul_t(h.view(B * T, D), wemb.t(), bemb, out=logits)
+    return logits.view(B, T, V), [acts, h]
+
+
+def t_gpt2_forward_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
+    return t_gpt2_forward_with_acts_t(params, y, y_mask, y_indices, train, p_gen_aux)[0]
+
+
+def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_aux=None):
+    """model_triton.py:2583-2593 + :2489-2521: gradient nest shaped like `params`."""
+    L = len(params) - 3
+    if not train:
+        p_gen_aux = [0] * (1 + 3 * L)
+    (layer_acts, x_last), h = acts
+    wemb, bemb = params[0]
+    V, D = wemb.shape
+    B, T = y.shape
+    N = B * T
+    dlog = dloss_dx.reshape(N, V)                                       # view for padded buffers
+    if dlog.stride(1) != 1:
+        dlog = dlog.contiguous()
+    h2d = h.view(N, D)
+    dbemb = colsum_t(dlog)
+    dwemb = matmul_t(dlog.t(), h2d)                                     # [V,D]  LM-head weight grad
+    dh = matmul_t(dlog, wemb)                                           # [N,D]
+    dx, (dlnfg, dlnfb) = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D))
+    layer_grads = [None] * L
+    for i in reversed(range(L)):
+        dx, layer_grads[i] = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train,
+                                                   p_gen_aux[1 + 3 * i:4 + 3 * i])
+    d = t_dropout_bkwd2_t(dx, None, train, p_gen_aux[0])                # [N,D]
+    # positional table: sum over the batch (model_triton.py:2518 with indices = arange(T))
+    dpos = torch.zeros_like(params[1][0])
+    dpos[:T] = colsum_t(d.view(B, T * D)).view(T, D)
+    # embedding: scatter-add rows by token id, times sqrt(D); tied with the LM head (:2591)
+    demb = torch.zeros((V, D), dtype=torch.float32, device=d.device)
+    demb.index_add_(0, y.reshape(-1).to(torch.int64), d.to(torch.float32))
+    dwemb = (dwemb.to(torch.float32) + demb * math.sqrt(D)).to(wemb.dtype)
+    return [[dwemb, dbemb], [dpos]] + layer_grads + [[dlnfg, dlnfb]]
