@@ -48,6 +48,76 @@ struct GemmArgs {
     int epilogue;
 };
 
+// A run of K panels [kt0, kt1) of one C tile.  FAST: straight-line vector loads (interior
+// tile, whole panels); otherwise the element-wise edge loader.  Written as one flat
+// function (no closures) so that the prefetch registers are plain SSA values.
+template <typename T, int AMODE, int BMODE, bool FAST>
+__device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM], char* __restrict__ smem, int row0,
+                                         int col0, int kbeg, int kend, int kt0, int kt1) {
+    constexpr int BK = BKB / (int)sizeof(T);
+    if (kt0 >= kt1) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int lr = lane & 31, lg = lane >> 5;
+    const T* A = (const T*)g.a;
+    const T* B = (const T*)g.b;
+    char* sA0 = smem;
+    char* sB0 = smem + 2 * BM * BKB;
+    TileLoader<T, AMODE, BM, GEMM_THREADS> la;
+    TileLoader<T, BMODE, BN, GEMM_THREADS> lb;
+#define GEMM_FETCH(KT)                                                        \
+    do {                                                                      \
+        const int k0__ = kbeg + (KT) * BK;                                    \
+        if constexpr (FAST) {                                                 \
+            la.load_fast(A, g.a_row, g.a_k, row0, k0__, tid);                 \
+            lb.load_fast(B, g.b_row, g.b_k, col0, k0__, tid);                 \
+        } else {                                                              \
+            la.load_edge(A, g.a_row, g.a_k, row0, g.n, k0__, kend, tid);      \
+            lb.load_edge(B, g.b_row, g.b_k, col0, g.m, k0__, kend, tid);      \
+        }                                                                     \
+    } while (0)
+    GEMM_FETCH(kt0);
+    la.store(sA0, tid);
+    lb.store(sB0, tid);
+    __syncthreads();
+    for (int kt = kt0; kt < kt1; ++kt) {
+        const int p = (kt - kt0) & 1;
+        // Straight-line body: the last step re-fetches its own panels (discarded) instead
+        // of branching, so the prefetch registers never cross a control-flow edge.
+        GEMM_FETCH(kt + 1 < kt1 ? kt + 1 : kt);
+        // Keep the copies of the next panels in flight across the MFMA block: without the
+        // fences the scheduler sinks the LDS stores (and their vmcnt waits) up here.
+        __builtin_amdgcn_sched_barrier(0);
+        const char* cA = sA0 + p * (BM * BKB);
+        const char* cB = sB0 + p * (BN * BKB);
+        // MFMA operands are double-buffered by hand: chunk c+1 is read from LDS while
+        // the MFMAs of chunk c run; the fences keep the reads from piling up at the top.
+        typename Frag<T>::type fa[2][TM], fb[2][TN];
+#define GEMM_READ_CHUNK(C, BUF)                                                                              \
+    do {                                                                                                     \
+        const int q__ = (C) * 2 + lg;                                                                        \
+        _Pragma("unroll") for (int t = 0; t < TM; ++t) fa[BUF][t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q__); \
+        _Pragma("unroll") for (int t = 0; t < TN; ++t) fb[BUF][t] = read_frag<T>(cB, wn * 96 + t * 32 + lr, q__); \
+    } while (0)
+        GEMM_READ_CHUNK(0, 0);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (c < 3) GEMM_READ_CHUNK(c + 1, (c + 1) & 1);
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) mma_chunk(acc[tn][tm], fb[c & 1][tn], fa[c & 1][tm]);  // A-role = B panel
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        la.store(sA0 + (p ^ 1) * (BM * BKB), tid);
+        lb.store(sB0 + (p ^ 1) * (BN * BKB), tid);
+        __syncthreads();
+    }
+#undef GEMM_FETCH
+#undef GEMM_READ_CHUNK
+}
+
 template <typename T, int AMODE, int BMODE>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
@@ -55,8 +125,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
     constexpr int STAGE_BYTES = (GEMM_THREADS / 64) * 64 * STAGE_PITCH;
     constexpr int SMEM_BYTES = STAGE_BYTES > TILE_BYTES ? STAGE_BYTES : TILE_BYTES;
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
-    auto sA = [&](int p) -> char* { return smem + p * (BM * BKB); };
-    auto sB = [&](int p) -> char* { return smem + 2 * BM * BKB + p * (BN * BKB); };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -84,9 +152,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
     const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
     const int nk = (kend - kbeg + BK - 1) / BK;
 
-    const T* A = (const T*)g.a;
-    const T* B = (const T*)g.b;
-
     f32x16 acc[TN][TM];
 #pragma unroll
     for (int i = 0; i < TN; ++i)
@@ -95,65 +160,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // A run of K panels [kt0, kt1): FAST = straight-line vector loads (interior tile, whole
-    // panels), otherwise the element-wise edge loader.
-    auto run = [&](auto fast_tag, int kt0, int kt1) {
-        constexpr bool FAST = decltype(fast_tag)::value;
-        if (kt0 >= kt1) return;
-        TileLoader<T, AMODE, BM, GEMM_THREADS> la;
-        TileLoader<T, BMODE, BN, GEMM_THREADS> lb;
-        auto fetch = [&](int kt) {
-            const int k0 = kbeg + kt * BK;
-            if constexpr (FAST) {
-                la.load_fast(A, g.a_row, g.a_k, row0, k0, tid);
-                lb.load_fast(B, g.b_row, g.b_k, col0, k0, tid);
-            } else {
-                la.load_edge(A, g.a_row, g.a_k, row0, g.n, k0, kend, tid);
-                lb.load_edge(B, g.b_row, g.b_k, col0, g.m, k0, kend, tid);
-            }
-        };
-        fetch(kt0);
-        la.store(sA(0), tid);
-        lb.store(sB(0), tid);
-        __syncthreads();
-        for (int kt = kt0; kt < kt1; ++kt) {
-            const int p = (kt - kt0) & 1;
-            const bool more = kt + 1 < kt1;
-            if (more) fetch(kt + 1);
-            const char* cA = sA(p);
-            const char* cB = sB(p);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int q = c * 2 + lg;
-                typename Frag<T>::type fa[TM], fb[TN];
-#pragma unroll
-                for (int t = 0; t < TM; ++t) fa[t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q);  // C rows    -> MFMA B
-#pragma unroll
-                for (int t = 0; t < TN; ++t) fb[t] = read_frag<T>(cB, wn * 96 + t * 32 + lr, q);  // C columns -> MFMA A
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-                    for (int tm = 0; tm < TM; ++tm) mma_chunk(acc[tn][tm], fb[tn], fa[tm]);
-            }
-            if (more) {
-                la.store(sA(p ^ 1), tid);
-                lb.store(sB(p ^ 1), tid);
-            }
-            __syncthreads();
-        }
-    };
     constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
     const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
     const int nk_full = (kend - kbeg) / BK;  // whole panels
     if constexpr (VECTOR_OK) {
         if (interior) {
-            run(std::true_type{}, 0, nk_full);
-            run(std::false_type{}, nk_full, nk);
+            gemm_run<T, AMODE, BMODE, true>(g, acc, smem, row0, col0, kbeg, kend, 0, nk_full);
+            gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, nk_full, nk);
         } else {
-            run(std::false_type{}, 0, nk);
+            gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
         }
     } else {
-        run(std::false_type{}, 0, nk);
+        gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
     }
 
     // ---- epilogue: per 32-column slab, stage the wave's 64x32 fp32 block in LDS, then

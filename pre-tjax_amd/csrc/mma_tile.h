@@ -35,6 +35,25 @@ __device__ __forceinline__ void mma_chunk(f32x16& acc, const f32x4& a, const f32
 //   GENERIC: element(row,k) = p[row*s_row + k*s_k]   scalar loads, any strides/alignment
 // Rows >= nrows and k >= kend read as zero.
 // ---------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Raw bits of element e of a 16-byte vector of T, and the reverse (used by the edge and
+// transposing paths; the staging registers are plain 4 x u32 vectors so that they are
+// always promoted to registers).
+template <typename T> __device__ __forceinline__ uint32_t vec_get(const u32x4& v, int e) {
+    if constexpr (sizeof(T) == 4) return v[e];
+    else return (v[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+}
+template <typename T> __device__ __forceinline__ void vec_set(u32x4& v, int e, uint32_t bits) {
+    if constexpr (sizeof(T) == 4) v[e] = bits;
+    else v[e >> 1] = (e & 1) ? ((v[e >> 1] & 0xffffu) | (bits << 16)) : ((v[e >> 1] & 0xffff0000u) | bits);
+}
+template <typename T> __device__ __forceinline__ uint32_t elem_bits(const T* p) {
+    if constexpr (sizeof(T) == 4) return *reinterpret_cast<const uint32_t*>(p);
+    else return *reinterpret_cast<const uint16_t*>(p);
+}
+
 template <typename T, int MODE, int ROWS, int THREADS>
 struct TileLoader {
     static constexpr int VEC = VecOf<T>::N;
@@ -50,38 +69,41 @@ struct TileLoader {
     static constexpr int NQ = (NBLK + NW - 1) / NW; // quads per thread
     static_assert(ROWS % (VEC * 8) == 0 && BK % 32 == 0, "panel shape");
     static constexpr int NREG = MODE == MNMAJOR ? NQ * 4 : NV;
-    Pack<T, VEC> r[NREG];
+    u32x4 r[NREG];
 
     // Interior panels: every vector is fully inside the operand; straight-line 16-byte loads
-    // (no predicates, no branches, so all of them stay in flight together).
+    // (no predicates, no branches, so all of them stay in flight together).  The address is
+    // split into a wave-uniform 64-bit part (scalar registers) and one 32-bit per-lane
+    // offset that does not change along K.
     __device__ __forceinline__ void load_fast(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int k0,
                                               int tid) {
         static_assert(MODE != GENERIC, "GENERIC panels have no vector path");
         if constexpr (MODE == KMAJOR) {
-            const T* base = p + (int64_t)(row0 + (tid >> 3)) * s_row + k0 + (tid & 7) * VEC;
+            const T* ub = p + (int64_t)row0 * s_row + k0;                       // uniform
+            const uint32_t loff = (uint32_t)(tid >> 3) * (uint32_t)s_row + (tid & 7) * VEC;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                if (ROWS % RP != 0 && (tid >> 3) + RP * i >= ROWS) break;
-                r[i] = *reinterpret_cast<const Pack<T, VEC>*>(base + (int64_t)(RP * i) * s_row);
+                if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS))
+                    r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row + loff);
             }
         } else {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
+            const T* ub = p + (int64_t)k0 * s_k + row0;                         // uniform
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = w + qi * NW;
-                if (NBLK % NW != 0 && b >= NBLK) break;
-                const int row = row0 + ((b % JB) * 8 + jc_lo) * VEC;
-                const int kq = k0 + ((b / JB) * 8 + kq_lo) * 4;
-                const T* base = p + (int64_t)kq * s_k + row;
+                if ((NBLK % NW == 0) || (b < NBLK)) {
+                    const uint32_t loff =
+                        (uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k + ((b % JB) * 8 + jc_lo) * VEC;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    r[qi * 4 + i] = *reinterpret_cast<const Pack<T, VEC>*>(base + (int64_t)i * s_k);
+                    for (int i = 0; i < 4; ++i)
+                        r[qi * 4 + i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)i * s_k + loff);
+                }
             }
         }
     }
 
-    // Edge panels and GENERIC operands: element-wise loads with the address clamped to
-    // the operand's first element when out of range (branch-free), zero-filled.
+    // Edge panels and GENERIC operands: element-wise loads, zero-filled out of range.
     __device__ __forceinline__ void load_edge(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int nrows,
                                               int k0, int kend, int tid) {
         if constexpr (MODE == KMAJOR || MODE == GENERIC) {
@@ -89,32 +111,33 @@ struct TileLoader {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int prow = (tid >> 3) + RP * i;
-                if (ROWS % RP != 0 && prow >= ROWS) break;
                 const int row = row0 + prow;
                 const int k = k0 + c * VEC;
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if ((ROWS % RP == 0 || prow < ROWS) && row < nrows) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const bool ok = row < nrows && k + e < kend;
-                    const T v = p[ok ? (int64_t)row * s_row + (int64_t)(k + e) * s_k : 0];
-                    r[i].v[e] = ok ? v : from_f32<T>(0.f);
+                    for (int e = 0; e < VEC; ++e)
+                        if (k + e < kend) vec_set<T>(v, e, elem_bits<T>(p + (int64_t)row * s_row + (int64_t)(k + e) * s_k));
                 }
+                r[i] = v;
             }
         } else {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = w + qi * NW;
-                if (NBLK % NW != 0 && b >= NBLK) break;
                 const int row = row0 + ((b % JB) * 8 + jc_lo) * VEC;
                 const int kq = k0 + ((b / JB) * 8 + kq_lo) * 4;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < 4; ++i) {
+                    u32x4 v = {0u, 0u, 0u, 0u};
+                    if ((NBLK % NW == 0 || b < NBLK) && kq + i < kend) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        const bool ok = kq + i < kend && row + e < nrows;
-                        const T v = p[ok ? (int64_t)(kq + i) * s_k + row + e : 0];
-                        r[qi * 4 + i].v[e] = ok ? v : from_f32<T>(0.f);
+                        for (int e = 0; e < VEC; ++e)
+                            if (row + e < nrows) vec_set<T>(v, e, elem_bits<T>(p + (int64_t)(kq + i) * s_k + row + e));
                     }
+                    r[qi * 4 + i] = v;
+                }
             }
         }
     }
@@ -125,24 +148,30 @@ struct TileLoader {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int row = (tid >> 3) + RP * i;
-                if (ROWS % RP != 0 && row >= ROWS) break;
-                *reinterpret_cast<Pack<T, VEC>*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
+                if ((ROWS % RP == 0) || (row < ROWS))
+                    *reinterpret_cast<u32x4*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
             }
         } else {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = w + qi * NW;
-                if (NBLK % NW != 0 && b >= NBLK) break;
-                const int prow = ((b % JB) * 8 + jc_lo) * VEC;
-                const int kb = ((b / JB) * 8 + kq_lo) * 4 * (int)sizeof(T);  // byte offset of the quad in the row
+                if ((NBLK % NW == 0) || (b < NBLK)) {
+                    const int prow = ((b % JB) * 8 + jc_lo) * VEC;
+                    const int kb = ((b / JB) * 8 + kq_lo) * 4 * (int)sizeof(T);  // byte offset of the quad in the row
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const int row = prow + e;
-                    Pack<T, 4> t;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) t.v[i] = r[qi * 4 + i].v[e];
-                    *reinterpret_cast<Pack<T, 4>*>(lds + row * BKB + (((kb >> 4) ^ sw(row)) << 4) + (kb & 15)) = t;
+                    for (int e = 0; e < VEC; ++e) {
+                        const int row = prow + e;
+                        char* dst = lds + row * BKB + (((kb >> 4) ^ sw(row)) << 4) + (kb & 15);
+                        if constexpr (sizeof(T) == 4) {
+                            u32x4 t = {r[qi * 4 + 0][e], r[qi * 4 + 1][e], r[qi * 4 + 2][e], r[qi * 4 + 3][e]};
+                            *reinterpret_cast<u32x4*>(dst) = t;
+                        } else {
+                            u32x2 t = {vec_get<T>(r[qi * 4 + 0], e) | (vec_get<T>(r[qi * 4 + 1], e) << 16),
+                                       vec_get<T>(r[qi * 4 + 2], e) | (vec_get<T>(r[qi * 4 + 3], e) << 16)};
+                            *reinterpret_cast<u32x2*>(dst) = t;
+                        }
+                    }
                 }
             }
         }
