@@ -197,14 +197,42 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ d
     if ((threadIdx.x & 7) == 0 && row < T_) delta[(int64_t)bh * T_ + row] = s;
 }
 
+// ---- element-wise pieces (VALU budget: a wave64 VALU op costs 4 cycles, v_exp 16, and one
+//      K tile gives each lane 32 score elements against 16 MFMAs = 512 cycles; every
+//      instruction per element counts, so masks and dropout are compiled in only where used)
+constexpr float NEG_RAW = -8e9f;          // masked raw score: NEG_RAW * (1/sqrt(64)) = -1e9
+constexpr float MASKED_BELOW = -1e8f;     // log2-domain row max below this = fully masked row
+
+// Causal / explicit-mask visibility of the lane's 16 elements of sub-tile j written into
+// the raw scores (invisible -> NEG_RAW) and returned as a bit per element.
+//   pos0 = (lane's own index) - (first index of the sub-tile along registers) - 4*lg
+//   element i = 4a+b sits at register offset 8a+b: visible iff 8a+b <= pos0 (causal part).
+template <bool LANE_IS_QUERY>
+__device__ __forceinline__ uint32_t apply_causal(f32x16& s, int pos0) {
+    uint32_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int off = (i >> 2) * 8 + (i & 3);
+        // lane = query: key offset must be <= query;  lane = key: query offset must be >= key
+        const bool ok = LANE_IS_QUERY ? (off <= pos0) : (off >= pos0);
+        s[i] = ok ? s[i] : NEG_RAW;
+        bits |= ok ? (1u << i) : 0u;
+    }
+    return bits;
+}
+
+__device__ __forceinline__ float and_bits(float v, int32_t m) { return __int_as_float(__float_as_int(v) & m); }
+// all-ones / all-zeros from bit `pos` of w
+__device__ __forceinline__ int32_t bit_mask(uint32_t w, int pos) { return __builtin_amdgcn_sbfe((int32_t)w, pos, 1); }
+
 // ---- forward -------------------------------------------------------------------------
 // grid (ceil(T/128), B*H); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
-template <typename T>
+template <typename T, bool HAS_MASK, bool TRAIN>
 __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 2 * X::NP * PANEL;  // K panels then V^T panels
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
-    __shared__ uint32_t sbits[MAX_BITWORDS];
+    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -224,34 +252,31 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
     int nkt = (q0 + 128) / 64;
     if (nkt > a.T / 64) nkt = a.T / 64;
 
+    // Flat code (no closures) keeps the prefetch registers plain SSA values; the last step
+    // re-fetches its own tile instead of branching.
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP];
     TileLoader<T, MNMAJOR, 64, ATT_THREADS> lv[X::NP];
-    auto fetch = [&](int kt) {
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lk[p].load_fast(Kb, a.k_rs, 1, kt * 64, p * X::EPP, tid);
-            lv[p].load_fast(Vb, 1, a.v_rs, 0, kt * 64 + p * X::EPP, tid);
-        }
-    };
-    auto stash = [&](int st) {
-        char* base = smem + st * STAGE;
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lk[p].store(base + p * PANEL, tid);
-            lv[p].store(base + (X::NP + p) * PANEL, tid);
-        }
-    };
+#define FWD_FETCH(KT)                                                                  \
+    _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
+        lk[p].load_fast(Kb, a.k_rs, 1, (KT) * 64, p * X::EPP, tid);                    \
+        lv[p].load_fast(Vb, 1, a.v_rs, 0, (KT) * 64 + p * X::EPP, tid);                \
+    }
+#define FWD_STASH(ST)                                                                  \
+    _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
+        lk[p].store(smem + (ST) * STAGE + p * PANEL, tid);                             \
+        lv[p].store(smem + (ST) * STAGE + (X::NP + p) * PANEL, tid);                   \
+    }
 
-    fetch(0);
-    if (a.train) {
+    FWD_FETCH(0)
+    if constexpr (TRAIN) {
         const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
         for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
     }
-    stash(0);
+    FWD_STASH(0)
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
-    float m_run = NEG2, l_run = 0.f;
+    float m_run = NEG_RAW * sc, l_run = 0.f;
     f32x16 o[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -260,8 +285,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
-        const bool more = kt + 1 < nkt;
-        if (more) fetch(kt + 1);
+        FWD_FETCH(kt + 1 < nkt ? kt + 1 : kt)
+        __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {   // some key of this tile is visible to some query of the wave
             const char* kp = smem + st * STAGE;
@@ -273,96 +298,84 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
                 for (int e = 0; e < 16; ++e) s[j][e] = 0.f;
             rows_x_frags<T>(s, kp, qf, lr, lg);
 
-            float p[2][16];
-            const bool diag = key0 + 63 > qw0;
-            float tmax = -INFINITY;
+            if (key0 + 63 > qw0) {   // tile touches the diagonal for this wave
+#pragma unroll
+                for (int j = 0; j < 2; ++j) apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
+            }
+            if constexpr (HAS_MASK) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
+                        const uint32_t m4 =
+                            *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+#pragma unroll
+                        for (int b = 0; b < 4; ++b)
+                            s[j][g4 * 4 + b] = ((m4 >> (8 * b)) & 0xffu) ? s[j][g4 * 4 + b] : NEG_RAW;
+                    }
+            }
+            float tmax = s[0][0];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
-                    uint32_t m4 = 0x01010101u;
-                    if (a.mask) m4 = *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        float v = s[j][g4 * 4 + b] * sc;
-                        bool ok = ((m4 >> (8 * b)) & 0xff) != 0;
-                        if (diag) ok = ok && (kb + b <= query);
-                        v = ok ? v : NEG2;
-                        p[j][g4 * 4 + b] = v;
-                        tmax = fmaxf(tmax, v);
-                    }
-                }
+                for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[j][i]);
             tmax = fmaxf(tmax, xor32(tmax));
-            const float m_new = fmaxf(m_run, tmax);
+            const float m_new = fmaxf(m_run, tmax * sc);
             const float alpha = fast_exp2(m_run - m_new);
+            float p[2][16];
             float lsum = 0.f;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float e = fast_exp2(p[j][i] - m_new);
+                    const float e = fast_exp2(fmaf(s[j][i], sc, -m_new));
                     p[j][i] = e;
                     lsum += e;
                 }
             lsum += xor32(lsum);
-            l_run = l_run * alpha + lsum;
+            l_run = fmaf(l_run, alpha, lsum);
             m_run = m_new;
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
-            if (a.train) {
+            if constexpr (TRAIN) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const uint32_t w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
 #pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        p[j][i] = ((w >> ((i >> 2) * 8 + (i & 3))) & 1u) ? p[j][i] : 0.f;
+                    for (int i = 0; i < 16; ++i) p[j][i] = and_bits(p[j][i], bit_mask(w, (i >> 2) * 8 + (i & 3)));
                 }
             }
             tp_x_regs(o, vp, p, lr, lg, T());
         }
-        if (more) stash(st ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        FWD_STASH(st ^ 1)
         __syncthreads();
     }
+#undef FWD_FETCH
+#undef FWD_STASH
 
     if (query < a.T) {
-        const float f = (a.train ? 1.0f : 0.9f) / l_run;
+        const float f = (TRAIN ? 1.0f : 0.9f) / l_run;
         store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, o, f, lg);
         if (lg == 0) {
-            a.ms[(int64_t)bh * a.T + query] = m_run == NEG2 ? NEG_NAT : m_run * LN2;
+            a.ms[(int64_t)bh * a.T + query] = m_run < MASKED_BELOW ? NEG_NAT : m_run * LN2;
             a.ls[(int64_t)bh * a.T + query] = l_run;
         }
     }
 }
 
-// Shared by both backward passes: probability and score-gradient of one element.
-//   v   : scaled score in log2 units (already masked to NEG2 where invisible)
-//   dpv : dP element;  keep: dropout keep bit (train) -- eval scales by 0.9
-// returns P (pre-dropout); writes pd (post-dropout P) and ds (unscaled dS).
-__device__ __forceinline__ void softmax_bwd_elem(float v, float dpv, bool visible, bool keep, int train, float m2,
-                                                 float linv, float delta, float& pd, float& ds) {
-    const float p = fast_exp2(v - m2) * linv;
-    if (train) {
-        pd = keep ? p : 0.f;
-        dpv = keep ? dpv : 0.f;
-    } else {
-        pd = 0.9f * p;
-        dpv = 0.9f * dpv;
-    }
-    ds = visible ? p * (dpv - delta) : 0.f;
-}
-
 // ---- backward pass 1: dK, dV ------------------------------------------------------------
 // grid (ceil(T/128), B*H); wave w owns keys key0 + 32w .. +31 (lane = key); query tiles of 64.
-template <typename T>
+template <typename T, bool HAS_MASK, bool TRAIN>
 __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 4 * X::NP * PANEL;  // Q, dO, Q^T, dO^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
     __shared__ __attribute__((aligned(16))) float sstat[2][3][64];  // m2, 1/l, delta per stage
-    __shared__ uint32_t sbits[MAX_BITWORDS];
+    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -386,37 +399,35 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lq[X::NP], ld[X::NP];
     TileLoader<T, MNMAJOR, 64, ATT_THREADS> lqt[X::NP], ldt[X::NP];
     float st_m = 0.f, st_l = 1.f, st_d = 0.f;
-    auto fetch = [&](int qt) {
-        const int q0 = qt * 64;
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lq[p].load_fast(Qb, a.q_rs, 1, q0, p * X::EPP, tid);
-            ld[p].load_fast(dOb, a.do_rs, 1, q0, p * X::EPP, tid);
-            lqt[p].load_fast(Qb, 1, a.q_rs, 0, q0 + p * X::EPP, tid);
-            ldt[p].load_fast(dOb, 1, a.do_rs, 0, q0 + p * X::EPP, tid);
-        }
-        if (tid < 64) {
-            const int64_t i = (int64_t)bh * a.T + q0 + tid;
-            st_m = a.ms[i];
-            st_l = a.ls[i];
-            st_d = a.delta[i];
-        }
-    };
-    auto stash = [&](int st) {
-        char* base = smem + st * STAGE;
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lq[p].store(base + p * PANEL, tid);
-            ld[p].store(base + (X::NP + p) * PANEL, tid);
-            lqt[p].store(base + (2 * X::NP + p) * PANEL, tid);
-            ldt[p].store(base + (3 * X::NP + p) * PANEL, tid);
-        }
-        if (tid < 64) {
-            sstat[st][0][tid] = st_m * LOG2E;
-            sstat[st][1][tid] = 1.0f / st_l;
-            sstat[st][2][tid] = st_d;
-        }
-    };
+    const int64_t stat0 = (int64_t)bh * a.T + (tid & 63);
+#define KV_FETCH(QT)                                                                   \
+    {                                                                                  \
+        const int q0__ = (QT) * 64;                                                    \
+        _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                            \
+            lq[p].load_fast(Qb, a.q_rs, 1, q0__, p * X::EPP, tid);                     \
+            ld[p].load_fast(dOb, a.do_rs, 1, q0__, p * X::EPP, tid);                   \
+            lqt[p].load_fast(Qb, 1, a.q_rs, 0, q0__ + p * X::EPP, tid);                \
+            ldt[p].load_fast(dOb, 1, a.do_rs, 0, q0__ + p * X::EPP, tid);              \
+        }                                                                              \
+        st_m = a.ms[stat0 + q0__];                                                     \
+        st_l = a.ls[stat0 + q0__];                                                     \
+        st_d = a.delta[stat0 + q0__];                                                  \
+    }
+#define KV_STASH(ST)                                                                   \
+    {                                                                                  \
+        char* base__ = smem + (ST) * STAGE;                                            \
+        _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                            \
+            lq[p].store(base__ + p * PANEL, tid);                                      \
+            ld[p].store(base__ + (X::NP + p) * PANEL, tid);                            \
+            lqt[p].store(base__ + (2 * X::NP + p) * PANEL, tid);                       \
+            ldt[p].store(base__ + (3 * X::NP + p) * PANEL, tid);                       \
+        }                                                                              \
+        if (tid < 64) {                                                                \
+            sstat[ST][0][tid] = st_m * LOG2E;                                          \
+            sstat[ST][1][tid] = 1.0f / st_l;                                           \
+            sstat[ST][2][tid] = st_d;                                                  \
+        }                                                                              \
+    }
 
     f32x16 dk[2], dv[2];
 #pragma unroll
@@ -425,20 +436,20 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
         for (int e = 0; e < 16; ++e) dk[t][e] = dv[t][e] = 0.f;
 
     if (qt0 < nqt) {
-        fetch(qt0);
-        if (a.train) {
+        KV_FETCH(qt0)
+        if constexpr (TRAIN) {
             const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
             for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
         }
-        stash(0);
+        KV_STASH(0)
     }
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
     for (int qt = qt0; qt < nqt; ++qt) {
         const int st = (qt - qt0) & 1;
-        const bool more = qt + 1 < nqt;
-        if (more) fetch(qt + 1);
+        KV_FETCH(qt + 1 < nqt ? qt + 1 : qt)
+        __builtin_amdgcn_sched_barrier(0);
         const int q0 = qt * 64;
         if (q0 + 63 >= kw0) {   // some query of the tile sees some key of the wave
             const char* base = smem + st * STAGE;
@@ -450,12 +461,28 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
             rows_x_frags<T>(s, base, kf, lr, lg);                          // S  [query][key]
             rows_x_frags<T>(dp, base + X::NP * PANEL, vf, lr, lg);         // dP [query][key]
 
+            uint32_t okbits[2] = {0xffffu, 0xffffu};
+            const bool masked = HAS_MASK || (q0 < kw0 + 31);
+            if (q0 < kw0 + 31) {   // tile touches the diagonal for this wave
+#pragma unroll
+                for (int j = 0; j < 2; ++j) okbits[j] = apply_causal<false>(s[j], key - q0 - j * 32 - lg * 4);
+            }
+            if constexpr (HAS_MASK) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int qq = q0 + j * 32 + (i >> 2) * 8 + lg * 4 + (i & 3);
+                        const bool ok = a.mask[((int64_t)bidx * a.T + qq) * a.T + krow] != 0;
+                        s[j][i] = ok ? s[j][i] : NEG_RAW;
+                        okbits[j] &= ok ? 0xffffffffu : ~(1u << i);
+                    }
+            }
             float pd[2][16], ds[2][16];
-            const bool diag = q0 < kw0 + 31;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t w = 0xffffffffu;
-                if (a.train) w = keep_window(sbits, key + q0 + j * 32 + lg * 4);
+                uint32_t w = 0;
+                if constexpr (TRAIN) w = keep_window(sbits, key + q0 + j * 32 + lg * 4);
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const int qi = j * 32 + g4 * 8 + lg * 4;  // first of 4 consecutive queries (tile-relative)
@@ -465,22 +492,33 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         const int i = g4 * 4 + b;
-                        const int qq = q0 + qi + b;
-                        bool ok = true;
-                        if (a.mask) ok = a.mask[((int64_t)bidx * a.T + qq) * a.T + krow] != 0;
-                        if (diag) ok = ok && (key <= qq);
-                        const float v = ok ? s[j][i] * sc : NEG2;
-                        softmax_bwd_elem(v, dp[j][i], ok, (w >> (g4 * 8 + b)) & 1u, a.train, m4[b], l4[b], d4[b],
-                                         pd[j][i], ds[j][i]);
+                        const float p = fast_exp2(fmaf(s[j][i], sc, -m4[b])) * l4[b];
+                        float dsv;
+                        if constexpr (TRAIN) {
+                            const int32_t km = bit_mask(w, g4 * 8 + b);
+                            pd[j][i] = and_bits(p, km);
+                            dsv = p * (and_bits(dp[j][i], km) - d4[b]);
+                        } else {
+                            pd[j][i] = 0.9f * p;
+                            dsv = p * fmaf(dp[j][i], 0.9f, -d4[b]);
+                        }
+                        ds[j][i] = dsv;
                     }
+                }
+                if (masked) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
                 }
             }
             tp_x_regs(dv, base + 3 * X::NP * PANEL, pd, lr, lg, T());      // dV^T += dO^T P
             tp_x_regs(dk, base + 2 * X::NP * PANEL, ds, lr, lg, T());      // dK^T += Q^T dS
         }
-        if (more) stash(st ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        KV_STASH(st ^ 1)
         __syncthreads();
     }
+#undef KV_FETCH
+#undef KV_STASH
 
     if (key < a.T) {
         store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)key * a.out0_rs, dk, a.scale, lg);
@@ -490,12 +528,12 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
 
 // ---- backward pass 2: dQ ----------------------------------------------------------------
 // Same geometry as the forward (lane = query, key tiles of 64).
-template <typename T>
+template <typename T, bool HAS_MASK, bool TRAIN>
 __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 3 * X::NP * PANEL;  // K, V, K^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
-    __shared__ uint32_t sbits[MAX_BITWORDS];
+    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -521,30 +559,25 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP], lv[X::NP];
     TileLoader<T, MNMAJOR, 64, ATT_THREADS> lkt[X::NP];
-    auto fetch = [&](int kt) {
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lk[p].load_fast(Kb, a.k_rs, 1, kt * 64, p * X::EPP, tid);
-            lv[p].load_fast(Vb, a.v_rs, 1, kt * 64, p * X::EPP, tid);
-            lkt[p].load_fast(Kb, 1, a.k_rs, 0, kt * 64 + p * X::EPP, tid);
-        }
-    };
-    auto stash = [&](int st) {
-        char* base = smem + st * STAGE;
-#pragma unroll
-        for (int p = 0; p < X::NP; ++p) {
-            lk[p].store(base + p * PANEL, tid);
-            lv[p].store(base + (X::NP + p) * PANEL, tid);
-            lkt[p].store(base + (2 * X::NP + p) * PANEL, tid);
-        }
-    };
+#define DQ_FETCH(KT)                                                                   \
+    _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
+        lk[p].load_fast(Kb, a.k_rs, 1, (KT) * 64, p * X::EPP, tid);                    \
+        lv[p].load_fast(Vb, a.v_rs, 1, (KT) * 64, p * X::EPP, tid);                    \
+        lkt[p].load_fast(Kb, 1, a.k_rs, 0, (KT) * 64 + p * X::EPP, tid);               \
+    }
+#define DQ_STASH(ST)                                                                   \
+    _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
+        lk[p].store(smem + (ST) * STAGE + p * PANEL, tid);                             \
+        lv[p].store(smem + (ST) * STAGE + (X::NP + p) * PANEL, tid);                   \
+        lkt[p].store(smem + (ST) * STAGE + (2 * X::NP + p) * PANEL, tid);              \
+    }
 
-    fetch(0);
-    if (a.train) {
+    DQ_FETCH(0)
+    if constexpr (TRAIN) {
         const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
         for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
     }
-    stash(0);
+    DQ_STASH(0)
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
@@ -556,8 +589,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
-        const bool more = kt + 1 < nkt;
-        if (more) fetch(kt + 1);
+        DQ_FETCH(kt + 1 < nkt ? kt + 1 : kt)
+        __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {
             const char* base = smem + st * STAGE;
@@ -569,37 +602,68 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
             rows_x_frags<T>(s, base, qf, lr, lg);                        // S^T  [key][query]
             rows_x_frags<T>(dp, base + X::NP * PANEL, dof, lr, lg);      // dP^T [key][query]
 
+            uint32_t okbits[2] = {0xffffu, 0xffffu};
+            const bool masked = HAS_MASK || (key0 + 63 > qw0);
+            if (key0 + 63 > qw0) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) okbits[j] = apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
+            }
+            if constexpr (HAS_MASK) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
+                        const uint32_t m4 =
+                            *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const bool ok = ((m4 >> (8 * b)) & 0xffu) != 0;
+                            s[j][g4 * 4 + b] = ok ? s[j][g4 * 4 + b] : NEG_RAW;
+                            okbits[j] &= ok ? 0xffffffffu : ~(1u << (g4 * 4 + b));
+                        }
+                    }
+            }
             float ds[2][16];
-            const bool diag = key0 + 63 > qw0;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t w = 0xffffffffu;
-                if (a.train) w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
+                uint32_t w = 0;
+                if constexpr (TRAIN) w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
-                    uint32_t m4 = 0x01010101u;
-                    if (a.mask) m4 = *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+                for (int i = 0; i < 16; ++i) {
+                    const float p = fast_exp2(fmaf(s[j][i], sc, -m2)) * linv;
+                    if constexpr (TRAIN)
+                        ds[j][i] = p * (and_bits(dp[j][i], bit_mask(w, (i >> 2) * 8 + (i & 3))) - delta);
+                    else
+                        ds[j][i] = p * fmaf(dp[j][i], 0.9f, -delta);
+                }
+                if (masked) {
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const int i = g4 * 4 + b;
-                        bool ok = ((m4 >> (8 * b)) & 0xff) != 0;
-                        if (diag) ok = ok && (kb + b <= query);
-                        const float v = ok ? s[j][i] * sc : NEG2;
-                        float pd_unused;
-                        softmax_bwd_elem(v, dp[j][i], ok, (w >> (g4 * 8 + b)) & 1u, a.train, m2, linv, delta, pd_unused,
-                                         ds[j][i]);
-                    }
+                    for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
                 }
             }
             tp_x_regs(dq, base + 2 * X::NP * PANEL, ds, lr, lg, T());    // dQ^T += K^T dS^T
         }
-        if (more) stash(st ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        DQ_STASH(st ^ 1)
         __syncthreads();
     }
+#undef DQ_FETCH
+#undef DQ_STASH
 
-    if (query < a.T) store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, dq, a.scale, lg);
+    if (query < a.T)
+        store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, dq, a.scale, lg);
 }
+
+// Launch one of the (mask, train) specialisations.
+#define ATTN_LAUNCH(KERNEL, T_, grid, st, args)                                                        \
+    do {                                                                                               \
+        const bool hm__ = (args).mask != nullptr, tr__ = (args).train != 0;                            \
+        if (hm__ && tr__) hipLaunchKernelGGL((KERNEL<T_, true, true>), grid, dim3(ATT_THREADS), 0, st, args);        \
+        else if (hm__) hipLaunchKernelGGL((KERNEL<T_, true, false>), grid, dim3(ATT_THREADS), 0, st, args);          \
+        else if (tr__) hipLaunchKernelGGL((KERNEL<T_, false, true>), grid, dim3(ATT_THREADS), 0, st, args);          \
+        else hipLaunchKernelGGL((KERNEL<T_, false, false>), grid, dim3(ATT_THREADS), 0, st, args);                   \
+    } while (0)
 
 // ---- host side ----------------------------------------------------------------------------
 inline size_t bits_bytes(int64_t BH, int64_t T) { return (size_t)BH * (2 * T / 32 + 2) * sizeof(uint32_t); }
@@ -663,8 +727,8 @@ int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mas
         if (rc) return rc;
     }
     dim3 grid((unsigned)((T + 127) / 128), (unsigned)BH);
-    if (dtype == PTJ_F32) hipLaunchKernelGGL((attn_fwd_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a);
+    if (dtype == PTJ_F32) ATTN_LAUNCH(attn_fwd_kernel, float, grid, st, a);
+    else ATTN_LAUNCH(attn_fwd_kernel, bf16, grid, st, a);
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
 }
@@ -717,11 +781,11 @@ int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, c
     AttnArgs a2 = a;
     a2.out0 = dq; a2.out0_bs = dq_bs; a2.out0_hs = dq_hs; a2.out0_rs = dq_rs;
     if (dtype == PTJ_F32) {
-        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a1);
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<float>), grid, dim3(ATT_THREADS), 0, st, a2);
+        ATTN_LAUNCH(attn_bwd_dkdv_kernel, float, grid, st, a1);
+        ATTN_LAUNCH(attn_bwd_dq_kernel, float, grid, st, a2);
     } else {
-        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a1);
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<bf16>), grid, dim3(ATT_THREADS), 0, st, a2);
+        ATTN_LAUNCH(attn_bwd_dkdv_kernel, bf16, grid, st, a1);
+        ATTN_LAUNCH(attn_bwd_dq_kernel, bf16, grid, st, a2);
     }
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
