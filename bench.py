@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--steps-only", action="store_true",
+                    help="only the timed training steps (for profiling): no per-kernel legs, no CPU leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards by batch; see DESIGN.md); "
@@ -104,6 +106,10 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     value = args.steps / dt
+    if args.steps_only:
+        print(json.dumps({"value": round(value, 4), "unit": "it/s", "ms_per_step": round(ms_per_step, 3),
+                          "steps": args.steps, "warmup": args.warmup}))
+        return
 
     # ---- second pass over further steps with HIP events around every GEMM launch ----------
     ev = []
@@ -115,7 +121,7 @@ def main():
             s.record()
             rc = orig_gemm(*a)
             e.record()
-            ev.append((s, e, 2.0 * a[4] * a[5] * a[6]))
+            ev.append((s, e, 2.0 * a[4] * a[5] * a[6]))   # 2*n*m*k
             return rc
 
     _lib._lib.ptj_gemm = Timed()

@@ -129,12 +129,28 @@ int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64
  * 16 bytes take the vectorised path; anything else (any strides) is still computed,
  * through scalar loads.  `workspace` (nullable) lets small outputs with a long k be
  * split along k: pass ptj_gemm_workspace_bytes(n, m, k, dtype) bytes; the split
- * partials are reduced in fixed order, so results are deterministic. */
+ * partials are reduced in fixed order, so results are deterministic.  `c_pre`
+ * (nullable, PTJ_EPI_BIAS_GELU only) additionally receives A.B + bias before the GELU:
+ * the activation the backward needs (the reference recomputes it, model_triton.py:1415-1418). */
 size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype);
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
              int64_t n, int64_t m, int64_t k,
              int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs,
-             int epilogue, void* workspace, size_t workspace_bytes, int dtype, void* stream);
+             int epilogue, void* c_pre, int64_t c_pre_rs,
+             void* workspace, size_t workspace_bytes, int dtype, void* stream);
+
+/* ---- optimizer ----------------------------------------------------------- */
+
+/* Fused AdamW update of one tensor, in place on the fp32 master weight and moments
+ * (replaces the per-tensor Python loops of adam_w_in_place,
+ * loss_and_optimizer_triton.py:376-401): with step t = i+1,
+ *   m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;
+ *   p += -lr * ( (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps) + weight_decay * p ).
+ * `g` has grad_dtype (fp32 or bf16); `shadow` (nullable, shadow_dtype) receives the
+ * updated weight rounded to the compute type. */
+int ptj_adamw(float* p, float* m, float* v, const void* g, void* shadow, int64_t n,
+              float lr, float beta1, float beta2, float eps, float weight_decay, int64_t t,
+              int grad_dtype, int shadow_dtype, void* stream);
 
 /* ---- attention ----------------------------------------------------------- */
 

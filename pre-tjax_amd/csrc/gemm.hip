@@ -28,17 +28,21 @@
 
 namespace {
 
-constexpr int BM = 256, BN = 192;       // C tile (rows from A, columns from B)
-constexpr int GEMM_THREADS = 512;
-constexpr int WAVES_N = 2;              // 4 x 2 wavefronts, each 64 rows x 96 columns
+#ifndef PTJ_GEMM_BM
+#define PTJ_GEMM_BM 256
+#endif
+constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from B)
+constexpr int WAVES_N = 2;                  // (BM/64) x 2 wavefronts, each 64 rows x 96 columns
+constexpr int GEMM_THREADS = (BM / 64) * WAVES_N * 64;
 constexpr int TM = 2, TN = 3;           // 32x32 MFMA tiles per wavefront
-constexpr int STAGE_PITCH = 32 * 4 + 16;  // bytes per staged fp32 row of a 64x32 slab
 
 struct GemmArgs {
     const void* a;
     const void* b;
     void* c;
     const void* bias;
+    void* c_aux;      // optional second output: A.B + bias before the GELU (nullptr = none)
+    int64_t c_aux_rs;
     float* partial;   // split-K workspace [splits][n][m] (nullptr when splits == 1)
     int n, m, k;
     int64_t a_row, a_k;   // strides of A(row=n, k)
@@ -118,13 +122,80 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM
 #undef GEMM_READ_CHUNK
 }
 
+// Writes the wave's 64x96 accumulator block to `dst` (row pitch dst_rs elements of OUT),
+// ROWS (32 or 64) rows per pass through a wave-private LDS staging area.
+template <typename OUT, typename T, int ROWS, bool EPILOGUE, bool NO_ACT = false>
+__device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
+                                                 int row0, int col0, OUT* __restrict__ dst, int64_t dst_rs) {
+    constexpr int PITCH = 96 * (int)sizeof(OUT) + 16;            // bytes per staged row
+    constexpr int V = 16 / (int)sizeof(OUT);                     // elements per 16-byte vector
+    constexpr int VPR = 96 / V;                                  // vectors per row
+    static_assert((GEMM_THREADS / 64) * ROWS * PITCH <= 2 * (BM + BN) * BKB, "staging area");
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int lr = lane & 31, lg = lane >> 5;
+    char* stage = smem + wave * (ROWS * PITCH);
+    const int gcol0 = col0 + wn * 96;
+    const int grow0 = row0 + wm * 64;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) && (dst_rs % V == 0);
+#pragma unroll
+    for (int pass = 0; pass < 64 / ROWS; ++pass) {
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int cc = tn * 32 + i4 * 8 + lg * 4;        // first of 4 columns, block-relative
+                float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (EPILOGUE) {
+                    if (g.epilogue != PTJ_EPI_NONE) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (gcol0 + cc + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol0 + cc + e]);
+                    }
+                }
+#pragma unroll
+                for (int tmi = 0; tmi < ROWS / 32; ++tmi) {
+                    const int tm = pass * (ROWS / 32) + tmi;
+                    float o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        o[e] = acc[tn][tm][i4 * 4 + e];
+                        if constexpr (EPILOGUE) {
+                            o[e] += bias4[e];
+                            if (!NO_ACT && g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
+                        }
+                    }
+                    store_vec<OUT, 4>(reinterpret_cast<OUT*>(stage + (tmi * 32 + lr) * PITCH) + cc, o);
+                }
+            }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   // the wave re-reads only its own area
+#pragma unroll
+        for (int it = 0; it < ROWS * VPR / 64; ++it) {
+            const int v = it * 64 + lane;
+            const int r = v / VPR, c = (v % VPR) * V;
+            const int grow = grow0 + pass * ROWS + r;
+            const int gcol = gcol0 + c;
+            const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(stage + r * PITCH + c * (int)sizeof(OUT));
+            if (grow >= g.n || gcol >= g.m) continue;
+            OUT* p = dst + (int64_t)grow * dst_rs + gcol;
+            if (aligned && gcol + V <= g.m) {
+                *reinterpret_cast<Pack<OUT, V>*>(p) = val;
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (gcol + e < g.m) p[e] = val.v[e];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    }
+}
+
 template <typename T, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(GEMM_THREADS, BM == 128 ? 2 : 1) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
     constexpr int TILE_BYTES = 2 * (BM + BN) * BKB;             // 112 KiB of operand panels
-    constexpr int STAGE_BYTES = (GEMM_THREADS / 64) * 64 * STAGE_PITCH;
-    constexpr int SMEM_BYTES = STAGE_BYTES > TILE_BYTES ? STAGE_BYTES : TILE_BYTES;
-    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -174,62 +245,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
         gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
     }
 
-    // ---- epilogue: per 32-column slab, stage the wave's 64x32 fp32 block in LDS, then
-    //      write rows back with contiguous stores.
-    // acc[tn][tm][i] of lane (lr, lg) = C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)]
-    char* stage = smem + wave * (64 * STAGE_PITCH);
-    const int cc4 = (lane & 7) * 4;  // 4 consecutive columns of the slab
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                f32x4 v = {acc[tn][tm][i4 * 4 + 0], acc[tn][tm][i4 * 4 + 1], acc[tn][tm][i4 * 4 + 2],
-                           acc[tn][tm][i4 * 4 + 3]};
-                *reinterpret_cast<f32x4*>(stage + (tm * 32 + lr) * STAGE_PITCH + (i4 * 8 + lg * 4) * 4) = v;
-            }
-        __syncthreads();
-        const int gcol = col0 + wn * 96 + tn * 32 + cc4;
-        float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-        if (g.epilogue != PTJ_EPI_NONE && g.partial == nullptr) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (gcol + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol + e]);
-        }
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const int r = (lane >> 3) + 8 * it;
-            const int grow = row0 + wm * 64 + r;
-            f32x4 v = *reinterpret_cast<const f32x4*>(stage + r * STAGE_PITCH + cc4 * 4);
-            if (grow >= g.n || gcol >= g.m) continue;
-            if (g.partial != nullptr) {
-                float* dst = g.partial + ((int64_t)blockIdx.z * g.n + grow) * g.m + gcol;
-                if (gcol + 4 <= g.m && (((uintptr_t)dst & 15) == 0)) {
-                    *reinterpret_cast<f32x4*>(dst) = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (gcol + e < g.m) dst[e] = v[e];
-                }
-                continue;
-            }
-            float o[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                o[e] = v[e] + bias4[e];
-                if (g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
-            }
-            T* dst = (T*)g.c + (int64_t)grow * g.c_rs + gcol;
-            if (gcol + 4 <= g.m && (((uintptr_t)dst & (4 * sizeof(T) - 1)) == 0)) {
-                store_vec<T, 4>(dst, o);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (gcol + e < g.m) dst[e] = from_f32<T>(o[e]);
-            }
-        }
-        __syncthreads();
+    // ---- epilogue.  acc[tn][tm][i] of lane (lr, lg) is
+    //   C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)].
+    // Bias / GELU are applied in registers, the block is converted to the output type and
+    // staged in a wave-private LDS area ([rows][96 columns]), then written back as 16-byte
+    // vectors that run along whole 96-column rows.  Only wave-local ordering is needed.
+    if (g.partial != nullptr) {
+        // split-K partial sums: fp32, one 32-row half at a time
+        gemm_store_block<float, T, 32, false>(g, acc, smem, row0, col0,
+                                              g.partial + (int64_t)blockIdx.z * g.n * (int64_t)g.m, g.m);
+    } else {
+        if (g.c_aux != nullptr)
+            gemm_store_block<T, T, sizeof(T) == 2 ? 64 : 32, true, true>(g, acc, smem, row0, col0, (T*)g.c_aux,
+                                                                         g.c_aux_rs);
+        gemm_store_block<T, T, sizeof(T) == 2 ? 64 : 32, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
     }
 }
 
@@ -237,13 +266,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial, int splits, int n,
                                                                   int m, T* __restrict__ c, int64_t c_rs,
-                                                                  const T* __restrict__ bias, int epilogue) {
+                                                                  const T* __restrict__ bias, int epilogue,
+                                                                  T* __restrict__ c_aux, int64_t c_aux_rs) {
     const int64_t total = (int64_t)n * m;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         float s = 0.f;
         for (int z = 0; z < splits; ++z) s += partial[z * total + i];
         const int row = (int)(i / m), col = (int)(i - (int64_t)row * m);
         if (epilogue != PTJ_EPI_NONE) s += to_f32(bias[col]);
+        if (c_aux != nullptr) c_aux[(int64_t)row * c_aux_rs + col] = from_f32<T>(s);
         if (epilogue == PTJ_EPI_BIAS_GELU) s = gelu_f(s);
         c[(int64_t)row * c_rs + col] = from_f32<T>(s);
     }
@@ -282,7 +313,8 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
         int64_t blocks = (total + 255) / 256;
         if (blocks > 256 * 8) blocks = 256 * 8;
         hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st,
-                           (const float*)g.partial, splits, g.n, g.m, (T*)g.c, g.c_rs, (const T*)g.bias, g.epilogue);
+                           (const float*)g.partial, splits, g.n, g.m, (T*)g.c, g.c_rs, (const T*)g.bias, g.epilogue,
+                           (T*)g.c_aux, g.c_aux_rs);
         PTJ_CHECK_LAUNCH();
     }
     return PTJ_OK;
@@ -313,8 +345,8 @@ size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype) {
 }
 
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n, int64_t m, int64_t k, int64_t a_rs,
-             int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs, int epilogue, void* workspace,
-             size_t workspace_bytes, int dtype, void* stream) {
+             int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs, int epilogue, void* c_pre, int64_t c_pre_rs,
+             void* workspace, size_t workspace_bytes, int dtype, void* stream) {
     PTJ_CHECK_ARG(n >= 0 && m >= 0 && k >= 0, "gemm: negative dimension");
     PTJ_CHECK_ARG(n < (1ll << 31) && m < (1ll << 31) && k < (1ll << 31), "gemm: dimension exceeds 31 bits");
     PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_BIAS_GELU, "gemm: unknown epilogue %d", epilogue);
@@ -323,6 +355,8 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     if (n == 0 || m == 0) return PTJ_OK;
     PTJ_CHECK_ARG(c && (k == 0 || (a && b)), "gemm: null pointer");
     PTJ_CHECK_ARG(c_rs >= m, "gemm: c row stride %lld < m %lld", (long long)c_rs, (long long)m);
+    PTJ_CHECK_ARG(!c_pre || (epilogue == PTJ_EPI_BIAS_GELU && c_pre_rs >= m),
+                  "gemm: c_pre needs the bias+GELU epilogue and a row stride >= m");
     const int elt = dtype == PTJ_BF16 ? 2 : 4;
     const int bk = BKB / elt;
     GemmArgs g;
@@ -331,6 +365,8 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     g.a_row = a_rs; g.a_k = a_cs;
     g.b_row = b_cs; g.b_k = b_rs;
     g.c_rs = c_rs;
+    g.c_aux = c_pre;
+    g.c_aux_rs = c_pre_rs;
     g.epilogue = epilogue;
     int splits = workspace ? choose_splits(n, m, k, elt, workspace_bytes) : 1;
     int64_t kps = k;

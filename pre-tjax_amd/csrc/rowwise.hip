@@ -400,7 +400,18 @@ __global__ __launch_bounds__(128) void colsum_stage1_kernel(const T* __restrict_
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int64_t r = r0; r < r1; ++r) {
+    constexpr int U = 8;   // independent row loads in flight per thread
+    int64_t r = r0;
+    for (; r + U <= r1; r += U) {
+        float v[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_vec<T, VEC>(x + (r + u) * xs + c0, v[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] += v[u][j];
+    }
+    for (; r < r1; ++r) {
         float v[VEC];
         load_vec<T, VEC>(x + r * xs + c0, v);
 #pragma unroll

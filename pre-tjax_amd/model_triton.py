@@ -194,12 +194,13 @@ def colsum_t(x: torch.Tensor):
 # ----------------------------------------------------------------------------------
 # GEMM  (reference: model_triton.py:373-398 t_matmul_t, :1258-1313 t_tlayer_ffn_fwd_t)
 # ----------------------------------------------------------------------------------
-def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None):
+def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, pre_out=None):
     """``out[N,M] = a[N,K] @ b[K,M] (+ bias[M]) (tanh-GELU)`` on the MFMA GEMM kernel.
 
     `a` and `b` are 2-D tensors with arbitrary strides (``.t()`` views are consumed in
     place, never copied); `out`, if given, is a 2-D tensor with unit column stride
-    (a column slice of a wider buffer is fine)."""
+    (a column slice of a wider buffer is fine).  `pre_out` (with ``gelu=True``) also
+    receives ``a @ b + bias`` before the activation."""
     require_gpu(a, b, bias, out)
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], (a.shape, b.shape)
     assert a.dtype == b.dtype
@@ -219,8 +220,11 @@ def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None):
     code = dtype_code(a)
     ws_bytes = lib().ptj_gemm_workspace_bytes(N, M, K, code)
     ws = _workspace(ws_bytes, a.device, "gemm") if ws_bytes else None
+    if pre_out is not None:
+        assert gelu and pre_out.shape == (N, M) and pre_out.dtype == a.dtype and pre_out.stride(1) == 1
     check(lib().ptj_gemm(ptr(a), ptr(b), ptr(out), ptr(bias), N, M, K, a.stride(0), a.stride(1), b.stride(0),
-                         b.stride(1), out.stride(0), epi, ptr(ws), ws_bytes, code, stream()), "ptj_gemm")
+                         b.stride(1), out.stride(0), epi, ptr(pre_out), pre_out.stride(0) if pre_out is not None else 0,
+                         ptr(ws), ws_bytes, code, stream()), "ptj_gemm")
     return out
 
 
@@ -396,8 +400,8 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
     a_out = matmul_t(o2, wo.t())
     x_mid = dropout_add_t(a_out, x_in, train, p_gen_aux[1])
     h2 = t_layernorm_fwd_t((ln2g, ln2b), x_mid)
-    f1 = matmul_t(h2, w1.t(), b1)
-    g1 = t_gelu_fwd_t(f1)
+    f1 = torch.empty((N, w1.shape[0]), dtype=y.dtype, device=y.device)
+    g1 = matmul_t(h2, w1.t(), b1, gelu=True, pre_out=f1)               # bias + GELU epilogue, both kept
     f2 = matmul_t(g1, w2.t(), b2)
     x_out = dropout_add_t(f2, x_mid, train, p_gen_aux[2])
     acts = (x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1)

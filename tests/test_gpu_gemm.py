@@ -97,3 +97,15 @@ def test_gemm_strided_output_and_misaligned_inputs(mt, dtype):
     pa[1:] = a.to(DEV).reshape(-1)
     c = mt.matmul_t(pa[1:].view(70, 41), b.to(DEV))
     check(c, a, b, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_gelu_dual_output(mt, dtype):
+    g = gen(14)
+    x, w, b = randn(g, 300, 200, dtype=dtype), randn(g, 260, 200, dtype=dtype, std=0.1), randn(g, 260, dtype=dtype)
+    pre = torch.empty(300, 260, dtype=dtype, device=DEV)
+    act = mt.matmul_t(x.to(DEV), w.to(DEV).t(), b.to(DEV), gelu=True, pre_out=pre)
+    check(pre, x, w.t(), dtype, bias=b)
+    check(act, x, w.t(), dtype, bias=b, gelu=True)
+    # the activation is computed from the unrounded pre-activation, exactly as the single-output epilogue
+    assert torch.equal(act, mt.matmul_t(x.to(DEV), w.to(DEV).t(), b.to(DEV), gelu=True))
