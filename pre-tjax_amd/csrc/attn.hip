@@ -226,7 +226,7 @@ __device__ __forceinline__ float and_bits(float v, int32_t m) { return __int_as_
 __device__ __forceinline__ int32_t bit_mask(uint32_t w, int pos) { return __builtin_amdgcn_sbfe((int32_t)w, pos, 1); }
 
 // ---- forward -------------------------------------------------------------------------
-// grid (ceil(T/128), B*H); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
+// grid (B*H, ceil(T/128)); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
 template <typename T, bool HAS_MASK, bool TRAIN>
 __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
     typedef AT<T> X;
@@ -236,8 +236,11 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
-    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
-    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128;   // heavy (late) query tiles first
+    // grid (B*H, T/128): the batch-head index is the fast dispatch dimension and the query
+    // tiles go from the longest (last) to the shortest, so the workgroups that start last
+    // are the cheapest ones (causal work per tile grows with the query position).
+    const int bh = blockIdx.x, bidx = bh / a.H, hidx = bh % a.H;
+    const int q0 = (gridDim.y - 1 - blockIdx.y) * 128;
     const int qw0 = q0 + wave * 32;
     const int query = qw0 + lr;
     const int qrow = query < a.T ? query : a.T - 1;
@@ -368,7 +371,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 }
 
 // ---- backward pass 1: dK, dV ------------------------------------------------------------
-// grid (ceil(T/128), B*H); wave w owns keys key0 + 32w .. +31 (lane = key); query tiles of 64.
+// grid (B*H, ceil(T/128)); wave w owns keys key0 + 32w .. +31 (lane = key); query tiles of 64.
 template <typename T, bool HAS_MASK, bool TRAIN>
 __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     typedef AT<T> X;
@@ -379,8 +382,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
-    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
-    const int key0 = blockIdx.x * 128;
+    const int bh = blockIdx.x, bidx = bh / a.H, hidx = bh % a.H;
+    const int key0 = blockIdx.y * 128;                    // first key tiles see the most queries: heavy first
     const int kw0 = key0 + wave * 32;
     const int key = kw0 + lr;
     const int krow = key < a.T ? key : a.T - 1;
@@ -537,8 +540,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
-    const int bh = blockIdx.y, bidx = bh / a.H, hidx = bh % a.H;
-    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128;
+    const int bh = blockIdx.x, bidx = bh / a.H, hidx = bh % a.H;
+    const int q0 = (gridDim.y - 1 - blockIdx.y) * 128;    // longest query tiles first
     const int qw0 = q0 + wave * 32;
     const int query = qw0 + lr;
     const int qrow = query < a.T ? query : a.T - 1;
@@ -726,7 +729,7 @@ int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mas
         rc = launch_keepbits((uint32_t*)workspace, BH, a.bitwords, seed, st);
         if (rc) return rc;
     }
-    dim3 grid((unsigned)((T + 127) / 128), (unsigned)BH);
+    dim3 grid((unsigned)BH, (unsigned)((T + 127) / 128));
     if (dtype == PTJ_F32) ATTN_LAUNCH(attn_fwd_kernel, float, grid, st, a);
     else ATTN_LAUNCH(attn_fwd_kernel, bf16, grid, st, a);
     PTJ_CHECK_LAUNCH();
@@ -774,7 +777,7 @@ int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, c
         hipLaunchKernelGGL((attn_delta_kernel<bf16>), dgrid, dim3(256), 0, st, (const bf16*)d_o, (const bf16*)o, delta,
                            (int)T, (int)H, do_bs, do_hs, do_rs, o_bs, o_hs, o_rs);
     PTJ_CHECK_LAUNCH();
-    dim3 grid((unsigned)((T + 127) / 128), (unsigned)BH);
+    dim3 grid((unsigned)BH, (unsigned)((T + 127) / 128));
     AttnArgs a1 = a;
     a1.out0 = dk; a1.out0_bs = dk_bs; a1.out0_hs = dk_hs; a1.out0_rs = dk_rs;
     a1.out1 = dv; a1.out1_bs = dv_bs; a1.out1_hs = dv_hs; a1.out1_rs = dv_rs;
