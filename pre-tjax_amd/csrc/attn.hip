@@ -74,8 +74,17 @@ __device__ __forceinline__ void load_row_frags(typename AT<T>::F (&f)[AT<T>::NC]
         f[c] = *reinterpret_cast<const typename AT<T>::F*>(reinterpret_cast<const char*>(row) + c * 32 + lg * 16);
 }
 
-// s[j] += panel_rows(j*32 + lr) x register_rows : panel rows become MFMA rows (m), the
+// s += panel_rows(j*32 + lr) x register_rows : panel rows become MFMA rows (m), the
 // lane's register row the MFMA column (n); contraction over the 64-element axis d.
+template <typename T>
+__device__ __forceinline__ void rows_x_frags_one(f32x16& s, const char* __restrict__ panels,
+                                                 const typename AT<T>::F (&f)[AT<T>::NC], int j, int lr, int lg) {
+#pragma unroll
+    for (int c = 0; c < AT<T>::NC; ++c) {
+        typename AT<T>::F a = read_frag<T>(panels + (c / 4) * PANEL, j * 32 + lr, (c % 4) * 2 + lg);
+        mma_chunk(s, a, f[c]);
+    }
+}
 template <typename T>
 __device__ __forceinline__ void rows_x_frags(f32x16 (&s)[2], const char* __restrict__ panels,
                                              const typename AT<T>::F (&f)[AT<T>::NC], int lr, int lg) {
@@ -91,43 +100,44 @@ __device__ __forceinline__ void rows_x_frags(f32x16 (&s)[2], const char* __restr
     }
 }
 
-// o[t] += transposed_panel_rows(t*32 + lr) x p : contraction over the 64 positions whose
-// values p[j][i] the lane holds in accumulator order (position = j*32 + 8*(i/4) + 4*lg + i%4).
-__device__ __forceinline__ void tp_x_regs(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[2][16],
-                                          int lr, int lg, bf16) {
+// o[t] += transposed_panel_rows(t*32 + lr) x p : contraction over the 32 positions of
+// sub-tile j whose values p[i] the lane holds in accumulator order
+// (position = j*32 + 8*(i/4) + 4*lg + i%4).
+__device__ __forceinline__ void tp_x_regs_one(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[16],
+                                              int j, int lr, int lg, bf16) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int h = 0; h < 2; ++h) {
+        bf16x8 b;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            bf16x8 b;
+        for (int e = 0; e < 8; ++e) b[e] = (bf16)p[8 * h + e];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) b[e] = (bf16)p[j][8 * h + e];
+        for (int t = 0; t < 2; ++t) {
+            const int row = t * 32 + lr;
+            const char* rp = panels + row * BKB + lg * 8;
+            const bf16x4 lo = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h) ^ sw(row)) << 4));
+            const bf16x4 hi = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h + 1) ^ sw(row)) << 4));
+            const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, o[t], 0, 0, 0);
+        }
+    }
+}
+__device__ __forceinline__ void tp_x_regs_one(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[16],
+                                              int j, int lr, int lg, float) {
+    const char* pp = panels + j * PANEL;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const int row = t * 32 + lr;
-                const char* rp = panels + row * BKB + lg * 8;
-                const bf16x4 lo = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h) ^ sw(row)) << 4));
-                const bf16x4 hi = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h + 1) ^ sw(row)) << 4));
-                const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, o[t], 0, 0, 0);
-            }
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const f32x4 v = read_frag<float>(pp, t * 32 + lr, 2 * a + lg);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[b], p[4 * a + b], o[t], 0, 0, 0);
         }
 }
+template <typename T>
 __device__ __forceinline__ void tp_x_regs(f32x16 (&o)[2], const char* __restrict__ panels, const float (&p)[2][16],
-                                          int lr, int lg, float) {
+                                          int lr, int lg, T tag) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const char* pp = panels + j * PANEL;
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const f32x4 v = read_frag<float>(pp, t * 32 + lr, 2 * a + lg);
-#pragma unroll
-                for (int b = 0; b < 4; ++b)
-                    o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[b], p[j][4 * a + b], o[t], 0, 0, 0);
-            }
-    }
+    for (int j = 0; j < 2; ++j) tp_x_regs_one(o, panels, p[j], j, lr, lg, tag);
 }
 
 // 32 keep bits starting at bit `ob` of the batch-head's bit line (LDS copy).
@@ -373,7 +383,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 // ---- backward pass 1: dK, dV ------------------------------------------------------------
 // grid (B*H, ceil(T/128)); wave w owns keys key0 + 32w .. +31 (lane = key); query tiles of 64.
 template <typename T, bool HAS_MASK, bool TRAIN>
-__global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 4 * X::NP * PANEL;  // Q, dO, Q^T, dO^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
@@ -456,34 +466,30 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
         const int q0 = qt * 64;
         if (q0 + 63 >= kw0) {   // some query of the tile sees some key of the wave
             const char* base = smem + st * STAGE;
-            f32x16 s[2], dp[2];
+            // The two 32-query halves are processed one after the other: half the live
+            // accumulators, which keeps two wavefronts per SIMD resident.
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 2; ++j) {
+                if (q0 + j * 32 + 31 < kw0) continue;   // every query of this half precedes the wave's keys
+                f32x16 s, dp;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) s[j][e] = dp[j][e] = 0.f;
-            rows_x_frags<T>(s, base, kf, lr, lg);                          // S  [query][key]
-            rows_x_frags<T>(dp, base + X::NP * PANEL, vf, lr, lg);         // dP [query][key]
+                for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
+                rows_x_frags_one<T>(s, base, kf, j, lr, lg);                      // S  [query][key]
+                rows_x_frags_one<T>(dp, base + X::NP * PANEL, vf, j, lr, lg);     // dP [query][key]
 
-            uint32_t okbits[2] = {0xffffu, 0xffffu};
-            const bool masked = HAS_MASK || (q0 < kw0 + 31);
-            if (q0 < kw0 + 31) {   // tile touches the diagonal for this wave
-#pragma unroll
-                for (int j = 0; j < 2; ++j) okbits[j] = apply_causal<false>(s[j], key - q0 - j * 32 - lg * 4);
-            }
-            if constexpr (HAS_MASK) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
+                uint32_t okbits = 0xffffu;
+                const bool diag = q0 + j * 32 < kw0 + 31;
+                if (diag) okbits = apply_causal<false>(s, key - q0 - j * 32 - lg * 4);
+                if constexpr (HAS_MASK) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int qq = q0 + j * 32 + (i >> 2) * 8 + lg * 4 + (i & 3);
                         const bool ok = a.mask[((int64_t)bidx * a.T + qq) * a.T + krow] != 0;
-                        s[j][i] = ok ? s[j][i] : NEG_RAW;
-                        okbits[j] &= ok ? 0xffffffffu : ~(1u << i);
+                        s[i] = ok ? s[i] : NEG_RAW;
+                        okbits &= ok ? 0xffffffffu : ~(1u << i);
                     }
-            }
-            float pd[2][16], ds[2][16];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
+                }
+                float pd[16], ds[16];
                 uint32_t w = 0;
                 if constexpr (TRAIN) w = keep_window(sbits, key + q0 + j * 32 + lg * 4);
 #pragma unroll
@@ -495,26 +501,24 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dkdv_kernel(const AttnAr
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         const int i = g4 * 4 + b;
-                        const float p = fast_exp2(fmaf(s[j][i], sc, -m4[b])) * l4[b];
-                        float dsv;
+                        const float p = fast_exp2(fmaf(s[i], sc, -m4[b])) * l4[b];
                         if constexpr (TRAIN) {
                             const int32_t km = bit_mask(w, g4 * 8 + b);
-                            pd[j][i] = and_bits(p, km);
-                            dsv = p * (and_bits(dp[j][i], km) - d4[b]);
+                            pd[i] = and_bits(p, km);
+                            ds[i] = p * (and_bits(dp[i], km) - d4[b]);
                         } else {
-                            pd[j][i] = 0.9f * p;
-                            dsv = p * fmaf(dp[j][i], 0.9f, -d4[b]);
+                            pd[i] = 0.9f * p;
+                            ds[i] = p * fmaf(dp[i], 0.9f, -d4[b]);
                         }
-                        ds[j][i] = dsv;
                     }
                 }
-                if (masked) {
+                if (HAS_MASK || diag) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
+                    for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
                 }
+                tp_x_regs_one(dv, base + 3 * X::NP * PANEL, pd, j, lr, lg, T());  // dV^T += dO^T P
+                tp_x_regs_one(dk, base + 2 * X::NP * PANEL, ds, j, lr, lg, T());  // dK^T += Q^T dS
             }
-            tp_x_regs(dv, base + 3 * X::NP * PANEL, pd, lr, lg, T());      // dV^T += dO^T P
-            tp_x_regs(dk, base + 2 * X::NP * PANEL, ds, lr, lg, T());      // dK^T += Q^T dS
         }
         __builtin_amdgcn_sched_barrier(0);
         KV_STASH(st ^ 1)
