@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="run one plain 1 GiB device copy first (reference reading for FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--steps-only", action="store_true",
                     help="only the timed training steps (for profiling): no per-kernel legs, no CPU leg")
     args = ap.parse_args()
@@ -96,6 +98,12 @@ def main():
         lo.adam_w_in_place(master, grads, 6e-4, (0.9, 0.95), 1e-8, moments, i, 0.1, wd_mask, shadow=shadow)
         losses.append(loss)
 
+    if args.copy_probe:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
