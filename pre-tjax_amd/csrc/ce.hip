@@ -26,6 +26,28 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restric
     }
 }
 
+// Writes one vector of the gradient row: subtracts 1/count at the label column (label < 0:
+// dead row) and stores, element-wise where the vector crosses a row boundary.  A plain
+// function rather than a closure so that `g` stays in registers.
+template <typename T>
+__device__ __forceinline__ void ce_emit(float (&g)[VecOf<T>::N], int vi, int mis, int cols, int64_t label,
+                                        float inv_cnt, T* __restrict__ db, T* __restrict__ dr) {
+    constexpr int VEC = VecOf<T>::N;
+    const int e0 = vi * VEC - mis;
+    const int64_t lj = label - e0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) g[j] -= (label >= 0 && lj == j) ? inv_cnt : 0.f;
+    if (e0 >= 0 && e0 + VEC <= cols) {
+        store_vec<T, VEC>(db + (int64_t)vi * VEC, g);
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const int e = e0 + j;
+            if (e >= 0 && e < cols) dr[e] = from_f32<T>(g[j]);
+        }
+    }
+}
+
 // CACHED: the row is kept in registers (ITERS vectors per thread).  Otherwise the
 // row is streamed from memory three times (max, sum, gradient).
 template <typename T, int ITERS, bool CACHED>
@@ -141,26 +163,6 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
         if (t == 0) row_loss[row] = live ? -(s_xy - m - logf(s)) : 0.f;
         const float scale = live ? inv_cnt / s : 0.f;
 
-        auto emit = [&](int vi, float (&g)[VEC]) {
-            const int e0 = vi * VEC - mis;
-            if (live) {
-                const int64_t lj = label - e0;
-                if (lj >= 0 && lj < VEC) {
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        if (j == (int)lj) g[j] -= inv_cnt;
-                }
-            }
-            if (e0 >= 0 && e0 + VEC <= cols) {
-                store_vec<T, VEC>(db + (int64_t)vi * VEC, g);
-            } else {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    const int e = e0 + j;
-                    if (e >= 0 && e < cols) dr[e] = from_f32<T>(g[j]);
-                }
-            }
-        };
         if constexpr (CACHED) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                     float g[VEC];
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) g[j] = v[it][j] * scale;
-                    emit(vi, g);
+                    ce_emit<T>(g, vi, mis, cols, live ? label : -1, inv_cnt, db, dr);
                 }
             }
         } else {
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                 load_vec<T, VEC>(xb + (int64_t)vi * VEC, g);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) g[j] = __expf(g[j] - m) * scale;
-                emit(vi, g);
+                ce_emit<T>(g, vi, mis, cols, live ? label : -1, inv_cnt, db, dr);
             }
         }
         __syncthreads();  // s_xy is rewritten by thread 0 at the top of the next row

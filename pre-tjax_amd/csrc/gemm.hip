@@ -321,16 +321,27 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
 }
 
 // Number of K splits for an (n, m, k) problem given `ws_bytes` of workspace.
+// Picks the split count that minimises a small cost model: the workgroups run in rounds
+// of one per CU, a workgroup costs a fixed prologue/epilogue plus a per-panel time, and
+// every split writes and re-reads an fp32 copy of C.
 int choose_splits(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes) {
+    constexpr int CUS = 256;
+    constexpr double T_FIXED_US = 6.0, T_PANEL_US = 1.6, BYTES_PER_US = 4.0e6;
     const int64_t tiles = ((n + BM - 1) / BM) * ((m + BN - 1) / BN);
     const int bk = BKB / elt;
-    if (tiles >= 256 || k < 16 * bk) return 1;
-    int64_t s = (512 + tiles - 1) / tiles;          // aim at ~2 workgroups per CU
-    const int64_t max_by_k = k / (8 * bk);          // at least 8 K-steps per split
-    if (s > max_by_k) s = max_by_k;
-    if (s > 32) s = 32;
-    while (s > 1 && (size_t)s * n * m * sizeof(float) > ws_bytes) --s;
-    return s < 1 ? 1 : (int)s;
+    const int64_t panels = (k + bk - 1) / bk;
+    if (tiles >= CUS || panels < 16) return 1;
+    int best = 1;
+    double best_cost = 0.0;
+    for (int s = 1; s <= 32; ++s) {
+        if (s > 1 && (panels / s < 8 || (size_t)s * n * m * sizeof(float) > ws_bytes)) break;
+        const int64_t rounds = (tiles * s + CUS - 1) / CUS;
+        const int64_t per_split = (panels + s - 1) / s;
+        double cost = (double)rounds * (T_FIXED_US + (double)per_split * T_PANEL_US);
+        if (s > 1) cost += 2.0 * (double)s * (double)n * (double)m * sizeof(float) / BYTES_PER_US;
+        if (s == 1 || cost < best_cost) { best = s; best_cost = cost; }
+    }
+    return best;
 }
 
 }  // namespace

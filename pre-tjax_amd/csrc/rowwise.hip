@@ -225,27 +225,44 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     }
 }
 
-// Second stage: out[which][c] = sum_p part[p][which][c], fixed order.
-// Block = 256 threads = 32 columns x 8 partial-slices; grid = (ceil(cols/32), 2).
-template <typename T>
-__global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float* __restrict__ part, int nparts,
-                                                                    int cols, T* __restrict__ dgamma,
-                                                                    T* __restrict__ dbeta) {
-    __shared__ float sm[8][33];
+// Sum over partials for one column, shared by the second-stage reducers: 1024 threads =
+// 32 columns x 32 slices; slice py adds partials py, py+32, ... (four independent chains so
+// that the loads overlap), then the slices are folded through LDS in slice order.
+constexpr int RED_THREADS = 1024;
+__device__ __forceinline__ float reduce_partials(const float* __restrict__ col_base, int64_t stride, int nparts,
+                                                 bool active, float (&sm)[32][33]) {
     const int cx = threadIdx.x & 31, py = threadIdx.x >> 5;
-    const int c = blockIdx.x * 32 + cx;
-    const int which = blockIdx.y;
-    float s = 0.f;
-    if (c < cols)
-        for (int p = py; p < nparts; p += 8) s += part[((int64_t)p * 2 + which) * cols + c];
-    sm[py][cx] = s;
-    __syncthreads();
-    if (py == 0 && c < cols) {
-        float r = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r += sm[i][cx];
-        (which == 0 ? dgamma : dbeta)[c] = from_f32<T>(r);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (active) {
+        int p = py;
+        for (; p + 96 < nparts; p += 128) {
+            s0 += col_base[(int64_t)p * stride];
+            s1 += col_base[(int64_t)(p + 32) * stride];
+            s2 += col_base[(int64_t)(p + 64) * stride];
+            s3 += col_base[(int64_t)(p + 96) * stride];
+        }
+        for (; p < nparts; p += 32) s0 += col_base[(int64_t)p * stride];
     }
+    sm[py][cx] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    float r = 0.f;
+    if (py == 0) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) r += sm[i][cx];
+    }
+    return r;
+}
+
+// Second stage: out[which][c] = sum_p part[p][which][c], fixed order.  grid = (ceil(cols/32), 2).
+template <typename T>
+__global__ __launch_bounds__(RED_THREADS) void layernorm_bwd_reduce_kernel(const float* __restrict__ part, int nparts,
+                                                                            int cols, T* __restrict__ dgamma,
+                                                                            T* __restrict__ dbeta) {
+    __shared__ float sm[32][33];
+    const int c = blockIdx.x * 32 + (threadIdx.x & 31);
+    const int which = blockIdx.y;
+    const float r = reduce_partials(part + (int64_t)which * cols + c, 2 * (int64_t)cols, nparts, c < cols, sm);
+    if ((threadIdx.x >> 5) == 0 && c < cols) (which == 0 ? dgamma : dbeta)[c] = from_f32<T>(r);
 }
 
 // ---------------------------------------------------------------------------------
@@ -422,27 +439,18 @@ __global__ __launch_bounds__(128) void colsum_stage1_kernel(const T* __restrict_
     for (int j = 0; j < VEC; ++j) dst[j] = acc[j];
 }
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_stage2_kernel(const float* __restrict__ part, int nparts, int cols,
-                                                            T* __restrict__ out) {
-    __shared__ float sm[8][33];
-    const int cx = threadIdx.x & 31, py = threadIdx.x >> 5;
-    const int c = blockIdx.x * 32 + cx;
-    float s = 0.f;
-    if (c < cols)
-        for (int p = py; p < nparts; p += 8) s += part[(int64_t)p * cols + c];
-    sm[py][cx] = s;
-    __syncthreads();
-    if (py == 0 && c < cols) {
-        float r = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r += sm[i][cx];
-        out[c] = from_f32<T>(r);
-    }
+__global__ __launch_bounds__(RED_THREADS) void colsum_stage2_kernel(const float* __restrict__ part, int nparts, int cols,
+                                                                     T* __restrict__ out) {
+    __shared__ float sm[32][33];
+    const int c = blockIdx.x * 32 + (threadIdx.x & 31);
+    const float r = reduce_partials(part + c, (int64_t)cols, nparts, c < cols, sm);
+    if ((threadIdx.x >> 5) == 0 && c < cols) out[c] = from_f32<T>(r);
 }
 
 inline void colsum_geometry(int64_t rows, int64_t cols, int vec, int* gx, int* splits, int* rps) {
     *gx = (int)((cols + 128 * vec - 1) / (128 * vec));
     int64_t s = 2048 / *gx;
+    if (s > 512) s = 512;
     if (s < 1) s = 1;
     if (s > (rows + 31) / 32) s = (rows + 31) / 32;
     if (s < 1) s = 1;
@@ -467,7 +475,7 @@ int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t row
         hipLaunchKernelGGL((colsum_stage1_kernel<T, 1>), dim3(gx, splits), dim3(128), 0, st, (const T*)x, (float*)ws,
                            rows, (int)cols, xs, rps);
     PTJ_CHECK_LAUNCH();
-    hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(256), 0, st,
+    hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
                        (const float*)ws, splits, (int)cols, (T*)out);
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
@@ -584,7 +592,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
 #undef LAUNCH_F
     PTJ_CHECK_LAUNCH();
     if (want_dgb) {
-        hipLaunchKernelGGL((layernorm_bwd_reduce_kernel<T>), dim3((unsigned)((cols + 31) / 32), 2), dim3(256), 0, st,
+        hipLaunchKernelGGL((layernorm_bwd_reduce_kernel<T>), dim3((unsigned)((cols + 31) / 32), 2), dim3(RED_THREADS), 0, st,
                            (const float*)ws, nparts, (int)cols, (T*)dgamma, (T*)dbeta);
         PTJ_CHECK_LAUNCH();
     }
