@@ -35,6 +35,16 @@ constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from
 constexpr int WAVES_N = 2;                  // (BM/64) x 2 wavefronts, each 64 rows x 96 columns
 constexpr int GEMM_THREADS = (BM / 64) * WAVES_N * 64;
 constexpr int TM = 2, TN = 3;           // 32x32 MFMA tiles per wavefront
+constexpr int NUM_CUS = 256;            // persistent grid: one workgroup per CU
+
+// threadIdx.x behind an opaque barrier: everything derived from it (LDS and global
+// offsets) is recomputed per call instead of being hoisted out of the persistent tile
+// loop, where it would stay live through every phase and spill.
+__device__ __forceinline__ int fresh_tid() {
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
 
 struct GemmArgs {
     const void* a;
@@ -49,18 +59,20 @@ struct GemmArgs {
     int64_t b_row, b_k;   // strides of B(row=m, k)  (b_row = b_cs, b_k = b_rs)
     int64_t c_rs;
     int k_per_split;      // multiple of BK
+    int splits;
+    int vec_out;          // every output (C, pre-activation, partials) and the bias allow aligned 16-byte rows
     int epilogue;
 };
 
-// A run of K panels [kt0, kt1) of one C tile.  FAST: straight-line vector loads (interior
-// tile, whole panels); otherwise the element-wise edge loader.  Written as one flat
+// A run of K panels [kt0, kt1) of one C tile through the element-wise edge loader (tiles
+// that cross the matrix border, partial panels, unaligned operands).  Written as one flat
 // function (no closures) so that the prefetch registers are plain SSA values.
-template <typename T, int AMODE, int BMODE, bool FAST>
+template <typename T, int AMODE, int BMODE>
 __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM], char* __restrict__ smem, int row0,
                                          int col0, int kbeg, int kend, int kt0, int kt1) {
     constexpr int BK = BKB / (int)sizeof(T);
     if (kt0 >= kt1) return;
-    const int tid = threadIdx.x;
+    const int tid = fresh_tid();
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int lr = lane & 31, lg = lane >> 5;
@@ -73,13 +85,8 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM
 #define GEMM_FETCH(KT)                                                        \
     do {                                                                      \
         const int k0__ = kbeg + (KT) * BK;                                    \
-        if constexpr (FAST) {                                                 \
-            la.load_fast(A, g.a_row, g.a_k, row0, k0__, tid);                 \
-            lb.load_fast(B, g.b_row, g.b_k, col0, k0__, tid);                 \
-        } else {                                                              \
-            la.load_edge(A, g.a_row, g.a_k, row0, g.n, k0__, kend, tid);      \
-            lb.load_edge(B, g.b_row, g.b_k, col0, g.m, k0__, kend, tid);      \
-        }                                                                     \
+        la.load_edge(A, g.a_row, g.a_k, row0, g.n, k0__, kend, tid);          \
+        lb.load_edge(B, g.b_row, g.b_k, col0, g.m, k0__, kend, tid);          \
     } while (0)
     GEMM_FETCH(kt0);
     la.store(sA0, tid);
@@ -122,143 +129,299 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM
 #undef GEMM_READ_CHUNK
 }
 
-// Writes the wave's 64x96 accumulator block to `dst` (row pitch dst_rs elements of OUT),
-// ROWS (32 or 64) rows per pass through a wave-private LDS staging area.
-template <typename OUT, typename T, int ROWS, bool EPILOGUE, bool NO_ACT = false>
-__device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
-                                                 int row0, int col0, OUT* __restrict__ dst, int64_t dst_rs) {
-    constexpr int PITCH = 96 * (int)sizeof(OUT) + 16;            // bytes per staged row
-    constexpr int V = 16 / (int)sizeof(OUT);                     // elements per 16-byte vector
-    constexpr int VPR = 96 / V;                                  // vectors per row
-    static_assert((GEMM_THREADS / 64) * ROWS * PITCH <= 2 * (BM + BN) * BKB, "staging area");
-    const int tid = threadIdx.x;
+// Whole K panels [0, nk) of an interior C tile, software-pipelined two panels deep:
+// while the MFMAs consume LDS buffer p (panel kt), panel kt+1 moves registers -> buffer
+// p^1 and panel kt+2 moves HBM -> registers.  A panel is four contraction chunks of six
+// MFMAs.  The instruction order is fixed by hand (every piece ends in a scheduling
+// fence): during chunks 0 and 1 the row-side operands of the next chunk are read up
+// front and each column-side operand is re-read right after its last use, with the
+// global loads and the LDS stores slotted between MFMA pairs; chunk 2 reads all of chunk
+// 3 first (the staging registers are free by then), so the single barrier of a step
+// finds no LDS read outstanding, and chunk 3 starts by reading chunk 0 of the other
+// buffer under its own MFMAs.  Loads past the last panel re-fetch it (discarded), so the
+// body has no branches and the staging registers stay plain values.
+template <typename T, int AMODE, int BMODE>
+__device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[TN][TM], char* __restrict__ smem,
+                                              int row0, int col0, int kbeg, int nk) {
+    constexpr int BK = BKB / (int)sizeof(T);
+    constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+    static_assert(TN == 3 && TM == 2, "the pipeline below is written for 2x3 MFMA tiles per wavefront");
+    if (nk <= 0) return;
+    const int tid = fresh_tid();
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int lr = lane & 31, lg = lane >> 5;
-    char* stage = smem + wave * (ROWS * PITCH);
+    const T* A = (const T*)g.a;
+    const T* B = (const T*)g.b;
+    char* sA = smem;
+    char* sB = smem + 2 * A_BYTES;
+    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1;
+    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1;
+    typename Frag<T>::type fa[2][TM], fb[TN], fx[TN];
+    const int last = nk - 1;
+    const int arow = wm * 64 + lr, brow = wn * 96 + lr;
+
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define K0_OF(KT) (kbeg + ((KT) < last ? (KT) : last) * BK)
+#define RD_A(P, C, BUF)                                                                                   \
+    do {                                                                                                  \
+        _Pragma("unroll") for (int t = 0; t < TM; ++t)                                                    \
+            fa[BUF][t] = read_frag<T>(sA + (P) * A_BYTES, arow + t * 32, (C) * 2 + lg);                   \
+    } while (0)
+#define RD_B(DST, P, C, TNI) DST = read_frag<T>(sB + (P) * B_BYTES, brow + (TNI) * 32, (C) * 2 + lg)
+#define MM(TNI, FB, BUF)                                                                                  \
+    do {                                                                                                  \
+        _Pragma("unroll") for (int tm = 0; tm < TM; ++tm) mma_chunk(acc[TNI][tm], FB, fa[BUF][tm]);       \
+    } while (0)
+    // One K step on buffer P.  LWA/LWB hold panel kt+1 (stored to buffer P^1), LFA/LFB
+    // receive panel KTF = kt+2.  On entry fa[0] and fb hold chunk 0 of buffer P.
+#define MV_A(I, LWA, LFA, P, KTF)                                                                         \
+    do {                                                                                                  \
+        LWA.template store_slice<I, 4>(sA + ((P) ^ 1) * A_BYTES, tid);                                    \
+        LFA.template load_fast_slice<I, 4>(A, g.a_row, g.a_k, row0, K0_OF(KTF), tid);                     \
+    } while (0)
+#define MV_B(I, LWB, LFB, P, KTF)                                                                         \
+    do {                                                                                                  \
+        LWB.template store_slice<I, 3>(sB + ((P) ^ 1) * B_BYTES, tid);                                    \
+        LFB.template load_fast_slice<I, 3>(B, g.b_row, g.b_k, col0, K0_OF(KTF), tid);                     \
+    } while (0)
+#define RF_STEP(P, LWA, LWB, LFA, LFB, KTF)                                                               \
+    do {                                                                                                  \
+        RD_A(P, 1, 1); SB();                                                                              \
+        MM(0, fb[0], 0); SB();                                                                            \
+        RD_B(fb[0], P, 1, 0); MV_A(0, LWA, LFA, P, KTF); SB();                                            \
+        MM(1, fb[1], 0); SB();                                                                            \
+        RD_B(fb[1], P, 1, 1); MV_A(1, LWA, LFA, P, KTF); SB();                                            \
+        MM(2, fb[2], 0); SB();                                                                            \
+        RD_B(fb[2], P, 1, 2); MV_A(2, LWA, LFA, P, KTF); SB();                                            \
+        RD_A(P, 2, 0); SB();                                                                              \
+        MM(0, fb[0], 1); SB();                                                                            \
+        RD_B(fb[0], P, 2, 0); MV_A(3, LWA, LFA, P, KTF); SB();                                            \
+        MM(1, fb[1], 1); SB();                                                                            \
+        RD_B(fb[1], P, 2, 1); MV_B(0, LWB, LFB, P, KTF); SB();                                            \
+        MM(2, fb[2], 1); SB();                                                                            \
+        RD_B(fb[2], P, 2, 2); MV_B(1, LWB, LFB, P, KTF); SB();                                            \
+        RD_A(P, 3, 1); RD_B(fx[0], P, 3, 0); RD_B(fx[1], P, 3, 1); RD_B(fx[2], P, 3, 2); SB();            \
+        MM(0, fb[0], 0); SB();                                                                            \
+        MV_B(2, LWB, LFB, P, KTF); SB();                                                                  \
+        MM(1, fb[1], 0); MM(2, fb[2], 0); SB();                                                           \
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                                   \
+        RD_A((P) ^ 1, 0, 0); RD_B(fb[0], (P) ^ 1, 0, 0); RD_B(fb[1], (P) ^ 1, 0, 1);                      \
+        RD_B(fb[2], (P) ^ 1, 0, 2); SB();                                                                 \
+        MM(0, fx[0], 1); MM(1, fx[1], 1); MM(2, fx[2], 1); SB();                                          \
+    } while (0)
+
+    la0.load_fast(A, g.a_row, g.a_k, row0, K0_OF(0), tid);
+    lb0.load_fast(B, g.b_row, g.b_k, col0, K0_OF(0), tid);
+    la1.load_fast(A, g.a_row, g.a_k, row0, K0_OF(1), tid);
+    lb1.load_fast(B, g.b_row, g.b_k, col0, K0_OF(1), tid);
+    la0.store(sA, tid);
+    lb0.store(sB, tid);
+    __syncthreads();
+    RD_A(0, 0, 0); RD_B(fb[0], 0, 0, 0); RD_B(fb[1], 0, 0, 1); RD_B(fb[2], 0, 0, 2); SB();
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+        RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+    }
+    if (kt < nk) RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+#undef SB
+#undef K0_OF
+#undef RD_A
+#undef RD_B
+#undef MM
+#undef RF_STEP
+#undef MV_A
+#undef MV_B
+}
+
+// LDS: two operand panel buffers (2 x 56 KiB) followed by one 6 KiB output staging area per
+// wavefront; the staging areas are separate from the panels so that a wavefront can write
+// its part of a finished tile while the others already load the next tile.
+constexpr int PANEL_BYTES = 2 * (BM + BN) * BKB;
+constexpr int STAGE_BYTES = 6144;
+constexpr int SMEM_BYTES = PANEL_BYTES + (GEMM_THREADS / 64) * STAGE_BYTES;
+
+// Writes the wave's 64x96 accumulator block to `dst` (row pitch dst_rs elements of OUT)
+// through the wave-private staging area: 32 rows per pass for 2-byte outputs, 16 for
+// 4-byte outputs.  A staged row is 96 outputs; its 16-byte chunks are rotated by the row
+// number (in place of padding) so that the 32 rows of a write land in different banks.
+// FULL: the tile lies inside C and dst / bias are vector-aligned, so the write-back is
+// straight-line 16-byte stores; otherwise every element is bounds-checked.  The two
+// variants are separate instantiations on purpose: when both appear behind one per-lane
+// condition the compiler merges them into partial (12 + 2 + 2 byte) stores.  The global
+// stores are not waited for.
+template <typename OUT, typename T, bool EPILOGUE, bool NO_ACT, bool FULL>
+__device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
+                                                 int row0, int col0, OUT* __restrict__ dst, int64_t dst_rs) {
+    constexpr int RB = 96 * (int)sizeof(OUT);                    // bytes per staged row
+    constexpr int NC = RB / 16;                                  // 16-byte chunks per row
+    constexpr int ROWS = STAGE_BYTES / RB;                       // rows per pass
+    constexpr int V = 16 / (int)sizeof(OUT);                     // elements per 16-byte vector
+    static_assert(ROWS == 32 || ROWS == 16, "staging pass");
+    const int tid = fresh_tid();
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int lr = lane & 31, lg = lane >> 5;
+    char* stage = smem + PANEL_BYTES + wave * STAGE_BYTES;
     const int gcol0 = col0 + wn * 96;
     const int grow0 = row0 + wm * 64;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) && (dst_rs % V == 0);
+    const int sr = lr & (ROWS - 1);                              // staged row of this lane
+    const int srot = sr % NC;
+    const bool has_bias = EPILOGUE && g.epilogue != PTJ_EPI_NONE;
+    const bool act = EPILOGUE && !NO_ACT && g.epilogue == PTJ_EPI_BIAS_GELU;
+
+    // bias of this lane's 12 column quads
+    float bias[TN * 4][4];
+    if constexpr (EPILOGUE) {
+#pragma unroll
+        for (int q = 0; q < TN * 4; ++q) {
+            const int cc = (q >> 2) * 32 + (q & 3) * 8 + lg * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bias[q][e] = 0.f;
+            if (has_bias) {
+                if constexpr (FULL) {
+                    load_vec<T, 4>((const T*)g.bias + gcol0 + cc, bias[q]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gcol0 + cc + e < g.m) bias[q][e] = to_f32(((const T*)g.bias)[gcol0 + cc + e]);
+                }
+            }
+        }
+    }
 #pragma unroll
     for (int pass = 0; pass < 64 / ROWS; ++pass) {
+        const int tm = pass * ROWS / 32;
+        const bool mine = ROWS == 32 || (lr >> 4) == (pass & 1);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int cc = tn * 32 + i4 * 8 + lg * 4;        // first of 4 columns, block-relative
-                float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = acc[tn][tm][i4 * 4 + e];
                 if constexpr (EPILOGUE) {
-                    if (g.epilogue != PTJ_EPI_NONE) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (gcol0 + cc + e < g.m) bias4[e] = to_f32(((const T*)g.bias)[gcol0 + cc + e]);
+                    for (int e = 0; e < 4; ++e) o[e] += bias[tn * 4 + i4][e];
+                    if (act) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = gelu_f(o[e]);
                     }
                 }
-#pragma unroll
-                for (int tmi = 0; tmi < ROWS / 32; ++tmi) {
-                    const int tm = pass * (ROWS / 32) + tmi;
-                    float o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        o[e] = acc[tn][tm][i4 * 4 + e];
-                        if constexpr (EPILOGUE) {
-                            o[e] += bias4[e];
-                            if (!NO_ACT && g.epilogue == PTJ_EPI_BIAS_GELU) o[e] = gelu_f(o[e]);
-                        }
-                    }
-                    store_vec<OUT, 4>(reinterpret_cast<OUT*>(stage + (tmi * 32 + lr) * PITCH) + cc, o);
-                }
+                const int byte = cc * (int)sizeof(OUT);
+                int ch = (byte >> 4) + srot;
+                ch = ch >= NC ? ch - NC : ch;
+                if (ROWS == 32 || mine)
+                    store_vec<OUT, 4>(reinterpret_cast<OUT*>(stage + sr * RB + (ch << 4) + (byte & 15)), o);
             }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   // the wave re-reads only its own area
 #pragma unroll
-        for (int it = 0; it < ROWS * VPR / 64; ++it) {
+        for (int it = 0; it < ROWS * NC / 64; ++it) {
             const int v = it * 64 + lane;
-            const int r = v / VPR, c = (v % VPR) * V;
+            const int r = v / NC, c = v % NC;
+            int ch = c + r % NC;
+            ch = ch >= NC ? ch - NC : ch;
             const int grow = grow0 + pass * ROWS + r;
-            const int gcol = gcol0 + c;
-            const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(stage + r * PITCH + c * (int)sizeof(OUT));
-            if (grow >= g.n || gcol >= g.m) continue;
+            const int gcol = gcol0 + c * V;
+            const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(stage + r * RB + (ch << 4));
             OUT* p = dst + (int64_t)grow * dst_rs + gcol;
-            if (aligned && gcol + V <= g.m) {
+            if constexpr (FULL) {
                 *reinterpret_cast<Pack<OUT, V>*>(p) = val;
             } else {
+                if (grow < g.n) {
 #pragma unroll
-                for (int e = 0; e < V; ++e)
-                    if (gcol + e < g.m) p[e] = val.v[e];
+                    for (int e = 0; e < V; ++e)
+                        if (gcol + e < g.m) p[e] = val.v[e];
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     }
 }
 
+// Persistent kernel: workgroup b handles work items b, b + gridDim.x, ... where an item is
+// one (C tile, K split) pair; the stores of a finished tile drain while the next tile's
+// panels are loaded and multiplied.
 template <typename T, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS, BM == 128 ? 2 : 1) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
-    constexpr int TILE_BYTES = 2 * (BM + BN) * BKB;             // 112 KiB of operand panels
-    __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
+    
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    const int lr = lane & 31, lg = lane >> 5;
-
-    // ---- workgroup -> tile ---------------------------------------------------------
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     const int total = num_m * num_n;
-    int pid = blockIdx.x;
-    {
-        const int chunk = total >> 3, rem = total & 7, x = pid & 7;
-        pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
-    }
-    constexpr int GROUP = 8;
-    const int width = GROUP * num_n;
-    const int group_id = pid / width;
-    const int first_m = group_id * GROUP;
-    const int gsz = (num_m - first_m) < GROUP ? (num_m - first_m) : GROUP;
-    const int tile_m = first_m + (pid % width) % gsz;
-    const int tile_n = (pid % width) / gsz;
-    const int row0 = tile_m * BM, col0 = tile_n * BN;
-
-    const int kbeg = blockIdx.z * g.k_per_split;
-    const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
-    const int nk = (kend - kbeg + BK - 1) / BK;
-
-    f32x16 acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
-    const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
-    const int nk_full = (kend - kbeg) / BK;  // whole panels
-    if constexpr (VECTOR_OK) {
-        if (interior) {
-            gemm_run<T, AMODE, BMODE, true>(g, acc, smem, row0, col0, kbeg, kend, 0, nk_full);
-            gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, nk_full, nk);
-        } else {
-            gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
+    const int work = total * g.splits;
+    for (int item = blockIdx.x; item < work; item += gridDim.x) {
+        const int z = item / total;
+        int pid = item - z * total;
+        // ---- work item -> tile: regroup so that the items of one XCD (id mod 8) cover a
+        // contiguous range of tiles, then walk groups of 8 tile-rows.
+        {
+            const int chunk = total >> 3, rem = total & 7, x = pid & 7;
+            pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
         }
-    } else {
-        gemm_run<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
-    }
+#ifndef PTJ_GEMM_GROUP
+#define PTJ_GEMM_GROUP 8
+#endif
+        constexpr int GROUP = PTJ_GEMM_GROUP;
+        const int width = GROUP * num_n;
+        const int group_id = pid / width;
+        const int first_m = group_id * GROUP;
+        const int gsz = (num_m - first_m) < GROUP ? (num_m - first_m) : GROUP;
+        const int tile_m = first_m + (pid % width) % gsz;
+        const int tile_n = (pid % width) / gsz;
+        const int row0 = tile_m * BM, col0 = tile_n * BN;
 
-    // ---- epilogue.  acc[tn][tm][i] of lane (lr, lg) is
-    //   C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)].
-    // Bias / GELU are applied in registers, the block is converted to the output type and
-    // staged in a wave-private LDS area ([rows][96 columns]), then written back as 16-byte
-    // vectors that run along whole 96-column rows.  Only wave-local ordering is needed.
-    if (g.partial != nullptr) {
-        // split-K partial sums: fp32, one 32-row half at a time
-        gemm_store_block<float, T, 32, false>(g, acc, smem, row0, col0,
-                                              g.partial + (int64_t)blockIdx.z * g.n * (int64_t)g.m, g.m);
-    } else {
-        if (g.c_aux != nullptr)
-            gemm_store_block<T, T, sizeof(T) == 2 ? 64 : 32, true, true>(g, acc, smem, row0, col0, (T*)g.c_aux,
-                                                                         g.c_aux_rs);
-        gemm_store_block<T, T, sizeof(T) == 2 ? 64 : 32, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        const int kbeg = z * g.k_per_split;
+        const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
+        const int nk = (kend - kbeg + BK - 1) / BK;
+
+        f32x16 acc[TN][TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+        constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
+        const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
+        const int nk_full = (kend - kbeg) / BK;  // whole panels
+        if constexpr (VECTOR_OK) {
+            if (interior) {
+                gemm_run_fast<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, nk_full);
+                if (nk_full < nk) {
+                    __syncthreads();   // the pipelined loop leaves LDS reads in flight
+                    gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, nk_full, nk);
+                }
+            } else {
+                gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
+            }
+        } else {
+            gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
+        }
+
+        // ---- epilogue.  acc[tn][tm][i] of lane (lr, lg) is
+        //   C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)].
+        // Bias / GELU are applied in registers, the block is converted to the output type,
+        // staged in the wave-private LDS area and written back as 16-byte vectors that run
+        // along whole 96-column rows.  Only wave-local ordering is needed.
+        const bool full = interior && g.vec_out;
+        if (g.partial != nullptr) {
+            float* part = g.partial + (int64_t)z * g.n * (int64_t)g.m;
+            if (full) gemm_store_block<float, T, false, false, true>(g, acc, smem, row0, col0, part, g.m);
+            else gemm_store_block<float, T, false, false, false>(g, acc, smem, row0, col0, part, g.m);
+        } else if (full) {
+            if (g.c_aux != nullptr)
+                gemm_store_block<T, T, true, true, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+            gemm_store_block<T, T, true, false, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        } else {
+            if (g.c_aux != nullptr)
+                gemm_store_block<T, T, true, true, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+            gemm_store_block<T, T, true, false, false>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        }
     }
 }
 
@@ -293,7 +456,8 @@ template <typename T>
 int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     const int am = pick_mode<T>(g.a, g.a_row, g.a_k), bm = pick_mode<T>(g.b, g.b_row, g.b_k);
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
-    dim3 grid(num_m * num_n, 1, splits), block(GEMM_THREADS);
+    const int64_t work = (int64_t)num_m * num_n * splits;
+    dim3 grid((unsigned)(work < NUM_CUS ? work : NUM_CUS)), block(GEMM_THREADS);
 #define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD>), grid, block, 0, st, g)
     switch (am * 3 + bm) {
         case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
@@ -387,6 +551,15 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     }
     if (kps < 1) kps = bk;  // k == 0: one empty pass writes bias / zeros
     g.k_per_split = (int)kps;
+    g.splits = splits;
+    {
+        const int64_t v = 16 / elt;
+        bool ok = ptj_aligned16(c) && c_rs % v == 0;
+        if (c_pre) ok = ok && ptj_aligned16(c_pre) && c_pre_rs % v == 0;
+        if (bias) ok = ok && (reinterpret_cast<uintptr_t>(bias) % (4 * (size_t)elt)) == 0;
+        if (splits > 1) ok = ok && ptj_aligned16(workspace) && m % 4 == 0;
+        g.vec_out = ok ? 1 : 0;
+    }
     g.partial = splits > 1 ? (float*)workspace : nullptr;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);

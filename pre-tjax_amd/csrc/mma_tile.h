@@ -11,7 +11,9 @@ constexpr int BKB = 128;  // bytes of the contraction axis per panel row
 
 enum LoadMode { KMAJOR = 0, MNMAJOR = 1, GENERIC = 2 };
 
-__device__ __forceinline__ int sw(int row) { return (row ^ (row >> 3)) & 7; }
+// Depends on row mod 32 only, so the rows of one lane's MFMA operands (32 apart) share a
+// swizzle and differ by a constant LDS offset.
+__device__ __forceinline__ int sw(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
 
 template <typename T> struct Frag;
 template <> struct Frag<bf16> { typedef bf16x8 type; };
@@ -54,7 +56,10 @@ template <typename T> __device__ __forceinline__ uint32_t elem_bits(const T* p) 
     else return *reinterpret_cast<const uint16_t*>(p);
 }
 
-template <typename T, int MODE, int ROWS, int THREADS>
+// WRAP (MNMAJOR only): when the 8x8 blocks do not divide evenly among the wavefronts, the
+// spare wavefronts repeat earlier blocks (same data to the same place) instead of idling,
+// which keeps the loader free of branches.
+template <typename T, int MODE, int ROWS, int THREADS, bool WRAP = false>
 struct TileLoader {
     static constexpr int VEC = VecOf<T>::N;
     static constexpr int BK = BKB / (int)sizeof(T);
@@ -77,27 +82,39 @@ struct TileLoader {
     // offset that does not change along K.
     __device__ __forceinline__ void load_fast(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int k0,
                                               int tid) {
+        load_fast_slice<0, 1>(p, s_row, s_k, row0, k0, tid);
+    }
+
+    // Slice I of N of load_fast (every N-th load), so that a caller can spread the loads of
+    // one panel between other work.
+    template <int I, int N>
+    __device__ __forceinline__ void load_fast_slice(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0,
+                                                    int k0, int tid) {
         static_assert(MODE != GENERIC, "GENERIC panels have no vector path");
+        // Byte addressing: wave-uniform 64-bit base + one unsigned 32-bit lane offset.
         if constexpr (MODE == KMAJOR) {
-            const T* ub = p + (int64_t)row0 * s_row + k0;                       // uniform
-            const uint32_t loff = (uint32_t)(tid >> 3) * (uint32_t)s_row + (tid & 7) * VEC;
+            const char* ub = reinterpret_cast<const char*>(p + (int64_t)row0 * s_row + k0);   // uniform
+            const uint32_t loff = ((uint32_t)(tid >> 3) * (uint32_t)s_row + (tid & 7) * VEC) * (uint32_t)sizeof(T);
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
+                if (i % N != I) continue;
                 if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS))
-                    r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row + loff);
+                    r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row * (int64_t)sizeof(T) + loff);
             }
         } else {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
-            const T* ub = p + (int64_t)k0 * s_k + row0;                         // uniform
+            const char* ub = reinterpret_cast<const char*>(p + (int64_t)k0 * s_k + row0);     // uniform
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
-                const int b = w + qi * NW;
-                if ((NBLK % NW == 0) || (b < NBLK)) {
-                    const uint32_t loff =
-                        (uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k + ((b % JB) * 8 + jc_lo) * VEC;
+                const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
+                if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
+                    const uint32_t loff = ((uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k +
+                                           ((b % JB) * 8 + jc_lo) * VEC) * (uint32_t)sizeof(T);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        r[qi * 4 + i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)i * s_k + loff);
+                    for (int i = 0; i < 4; ++i) {
+                        if ((qi * 4 + i) % N != I) continue;
+                        r[qi * 4 + i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)i * s_k * (int64_t)sizeof(T) + loff);
+                    }
                 }
             }
         }
@@ -125,13 +142,13 @@ struct TileLoader {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
-                const int b = w + qi * NW;
+                const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
                 const int row = row0 + ((b % JB) * 8 + jc_lo) * VEC;
                 const int kq = k0 + ((b / JB) * 8 + kq_lo) * 4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     u32x4 v = {0u, 0u, 0u, 0u};
-                    if ((NBLK % NW == 0 || b < NBLK) && kq + i < kend) {
+                    if ((WRAP || NBLK % NW == 0 || b < NBLK) && kq + i < kend) {
 #pragma unroll
                         for (int e = 0; e < VEC; ++e)
                             if (row + e < nrows) vec_set<T>(v, e, elem_bits<T>(p + (int64_t)(kq + i) * s_k + row + e));
@@ -142,11 +159,16 @@ struct TileLoader {
         }
     }
 
-    __device__ __forceinline__ void store(char* __restrict__ lds, int tid) const {
+    __device__ __forceinline__ void store(char* __restrict__ lds, int tid) const { store_slice<0, 1>(lds, tid); }
+
+    // Slice I of N of store (every N-th LDS write).
+    template <int I, int N>
+    __device__ __forceinline__ void store_slice(char* __restrict__ lds, int tid) const {
         if constexpr (MODE == KMAJOR || MODE == GENERIC) {
             const int c = tid & 7;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
+                if (i % N != I) continue;
                 const int row = (tid >> 3) + RP * i;
                 if ((ROWS % RP == 0) || (row < ROWS))
                     *reinterpret_cast<u32x4*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
@@ -155,12 +177,13 @@ struct TileLoader {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
-                const int b = w + qi * NW;
-                if ((NBLK % NW == 0) || (b < NBLK)) {
+                const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
+                if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
                     const int prow = ((b % JB) * 8 + jc_lo) * VEC;
                     const int kb = ((b / JB) * 8 + kq_lo) * 4 * (int)sizeof(T);  // byte offset of the quad in the row
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
+                        if ((qi * VEC + e) % N != I) continue;
                         const int row = prow + e;
                         char* dst = lds + row * BKB + (((kb >> 4) ^ sw(row)) << 4) + (kb & 15);
                         if constexpr (sizeof(T) == 4) {
