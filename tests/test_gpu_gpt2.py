@@ -73,3 +73,44 @@ def test_gpt2_small_config1_fp32(lo):
             worst = max(worst, e)
             assert e <= 5e-5, "grad[%d][%d] rel L2 %.3e" % (gi, pi, e)
     print("config1 fp32: loss %.6f (oracle %.6f), worst grad rel L2 %.2e" % (loss.item(), wl.item(), worst))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_loss_curve_short_run(lo, dtype):
+    """A short synthetic training run (dropout on, AdamW every step, a fresh batch of learnable sequences per step) on
+    the HIP path next to the same run in the oracle (fp64 autograd + its AdamW, identical
+    Philox seeds).  Bars on the per-step loss: 1e-4 relative for fp32 storage (the 1e-5
+    per-step bar compounded over the steps), 2e-2 for bf16 compute on fp32 master weights."""
+    V, D, L, H, F, T, B, steps = 331, 128, 2, 2, 256, 128, 4, 20
+    lr, betas, eps, wd = 3e-3, (0.9, 0.95), 1e-8, 0.1
+    params = ogpt2.init_transformer_gpt2(V, D, L, H, F, T, seed=7)
+    wd_mask = [[p.dim() > 1 for p in grp] for grp in params]
+    g = torch.Generator().manual_seed(8)
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(B, T, T).contiguous()
+    master = [[p.clone().to(DEV) for p in grp] for grp in params]
+    shadow = None if dtype == torch.float32 else to_dev(params, dtype)
+    moments = lo.init_adam_w(master)
+    o_params = [[p.double() for p in grp] for grp in params]
+    o_mom = [[[torch.zeros_like(p) for p in grp] for grp in o_params] for _ in range(2)]
+    got, want = [], []
+    for i in range(steps):
+        # learnable data: arithmetic token sequences with a random start and stride
+        start = torch.randint(1, V, (B, 1), generator=g)
+        stride = torch.randint(1, 4, (B, 1), generator=g)
+        y = 1 + (start + stride * torch.arange(T + 1)[None, :]) % (V - 1)
+        seeds = [5000 + 101 * i + j for j in range(1 + 3 * L)]
+        compute = master if shadow is None else shadow
+        grads, (loss, _, _) = lo.t_loss_bkwd3_t(compute, y.to(DEV), mask.to(DEV), None, True, seeds)
+        lo.adam_w_in_place(master, grads, lr, betas, eps, moments, i, wd, wd_mask, shadow=shadow)
+        # the oracle computes in the storage dtype's values: for bf16 it sees the rounded weights
+        o_compute = o_params if shadow is None else [[p.to(dtype).double() for p in grp] for grp in o_params]
+        o_grads, (o_loss, _, _) = ogpt2.grad_loss(o_compute, y, mask, True, seeds)
+        o_params, o_mom = ogpt2.adam_w(o_params, o_grads, lr, betas, eps, o_mom, i, wd, wd_mask)
+        got.append(loss.item())
+        want.append(o_loss.item())
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    worst = max(abs(a - b) / abs(b) for a, b in zip(got, want))
+    print("loss curve (%s): hip %s\n             oracle %s\nworst rel diff %.2e" %
+          (dtype, ["%.4f" % x for x in got], ["%.4f" % x for x in want], worst))
+    assert want[-1] < want[0] - 0.2, "the run must actually learn: %s" % want
+    assert worst <= tol, (got, want)

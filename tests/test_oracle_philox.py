@@ -61,9 +61,8 @@ def test_rowwise_mask_layout_and_rate():
 
 def test_attn_mask_depends_on_q_plus_k_only():
     m = philox.attn_keep_mask(3, 2, 8, 8)
-    for d in range(1, 8):
-        # moving one step along an anti-diagonal leaves q+k unchanged
-        assert (m[:, d:, :-d][:, 0, -1] == m[:, :, :][:, d - 1 + 1 - 1 + 0, 7 - d + 0 + 0][...]).all() or True
+    # moving one step along an anti-diagonal leaves q+k, and so the keep bit, unchanged
+    assert (m[:, 1:, :-1] == m[:, :-1, 1:]).all()
     q, k = np.meshgrid(np.arange(8), np.arange(8), indexing="ij")
     line = philox.tl_rand(np.int64(3 + 1), np.arange(15)) > np.float32(0.1)
     assert (m[1] == line[q + k]).all()
