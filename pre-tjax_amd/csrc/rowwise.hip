@@ -16,14 +16,15 @@ struct RowRegs {
     float v[ITERS][VEC];
     __device__ __forceinline__ void load(const T* __restrict__ row, int nvec, int t, float fill) {
 #pragma unroll
+        // Branch-free: lanes past the end of the row re-read its last vector and discard it,
+        // so that all loads of a row are in flight together (a load inside a per-lane branch
+        // is followed by a full wait).
         for (int it = 0; it < ITERS; ++it) {
             const int vi = t + it * TPR;
-            if (vi < nvec) {
-                load_vec<T, VEC>(row + (int64_t)vi * VEC, v[it]);
-            } else {
+            const int vc = vi < nvec ? vi : nvec - 1;
+            load_vec<T, VEC>(row + (int64_t)vc * VEC, v[it]);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) v[it][j] = fill;
-            }
+            for (int j = 0; j < VEC; ++j) v[it][j] = vi < nvec ? v[it][j] : fill;
         }
     }
     __device__ __forceinline__ void store(T* __restrict__ row, int nvec, int t) const {
@@ -122,9 +123,14 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     // Every thread of a >64-thread row group must take the same trip count because
     // row_reduce synchronises the block; with RPB == 1 all threads share `row`.
     for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
-        RowRegs<T, VEC, TPR, ITERS> r, d;
+        RowRegs<T, VEC, TPR, ITERS> r, d, rr;
         r.load(x + row * xs, nvec, t, 0.f);
         d.load(dy + row * dys, nvec, t, 0.f);
+        if constexpr (DX) {
+            // residual row, in flight under the reductions; without a residual the (cached)
+            // dy row is re-read and ignored, which keeps the load out of a branch
+            rr.load(res != nullptr ? res + row * (int64_t)cols : dy + row * dys, nvec, t, 0.f);
+        }
         float s = 0.f;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
@@ -172,11 +178,10 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
             if (res != nullptr) {
                 // residual branch: the sum is formed from the storage-rounded LayerNorm gradient,
                 // as two separate passes would
-                r.load(res + row * (int64_t)cols, nvec, t, 0.f);
 #pragma unroll
                 for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) d.v[it][j] = r.v[it][j] + to_f32(from_f32<T>(d.v[it][j]));
+                    for (int j = 0; j < VEC; ++j) d.v[it][j] = rr.v[it][j] + to_f32(from_f32<T>(d.v[it][j]));
             }
             d.store(dx + row * dxs, nvec, t);
         }
@@ -487,14 +492,16 @@ int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t row
 struct RowCfg {
     int vec;   // VEC or 1
     int tpr;   // 64, 256, 1024
+    int iters64;  // ITERS of the 64-thread row group: 1, 2 or 4
 };
 
 // Picks the smallest row-group that holds `cols` elements in registers.
-// ITERS is fixed per TPR: 64 -> 4, 256 -> 4, 1024 -> 8.
+// ITERS per TPR: 64 -> 1, 2 or 4 (the smallest that covers the row), 256 -> 4, 1024 -> 8.
 inline bool pick_row_cfg(int64_t cols, int full_vec, bool vec_ok, RowCfg* cfg) {
     const int vec = vec_ok ? full_vec : 1;
     const int64_t nvec = cols / vec;
     cfg->vec = vec;
+    cfg->iters64 = nvec <= 64 ? 1 : nvec <= 128 ? 2 : 4;
     if (nvec <= 64 * 4) cfg->tpr = 64;
     else if (nvec <= 256 * 4) cfg->tpr = 256;
     else if (nvec <= 1024 * 8) cfg->tpr = 1024;
@@ -513,11 +520,19 @@ inline int row_grid(int64_t rows, int tpr) {
     do {                                                                 \
         constexpr int FV = VecOf<T>::N;                                  \
         if (cfg.vec == 1) {                                              \
-            if (cfg.tpr == 64) { LAUNCH(T, 1, 64, 4); }                  \
+            if (cfg.tpr == 64) {                                         \
+                if (cfg.iters64 == 1) { LAUNCH(T, 1, 64, 1); }           \
+                else if (cfg.iters64 == 2) { LAUNCH(T, 1, 64, 2); }      \
+                else { LAUNCH(T, 1, 64, 4); }                            \
+            }                                                            \
             else if (cfg.tpr == 256) { LAUNCH(T, 1, 256, 4); }           \
             else { LAUNCH(T, 1, 1024, 8); }                              \
         } else {                                                         \
-            if (cfg.tpr == 64) { LAUNCH(T, FV, 64, 4); }                 \
+            if (cfg.tpr == 64) {                                         \
+                if (cfg.iters64 == 1) { LAUNCH(T, FV, 64, 1); }          \
+                else if (cfg.iters64 == 2) { LAUNCH(T, FV, 64, 2); }     \
+                else { LAUNCH(T, FV, 64, 4); }                           \
+            }                                                            \
             else if (cfg.tpr == 256) { LAUNCH(T, FV, 256, 4); }          \
             else { LAUNCH(T, FV, 1024, 8); }                             \
         }                                                                \
