@@ -10,6 +10,15 @@ namespace {
 
 constexpr int CE_THREADS = 1024;
 
+typedef uint32_t ce_u32x4 __attribute__((ext_vector_type(4)));
+
+// Asynchronous copy of 16 bytes per lane from global memory straight into LDS: lane l of a
+// wavefront lands at lds_wave_base + 16*l (the destination is wave-uniform by construction).
+__device__ __forceinline__ void ce_load_to_lds(const void* gsrc, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
 __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restrict__ labels, int64_t rows,
                                                          int64_t* __restrict__ count) {
     __shared__ int sm[16];
@@ -48,6 +57,25 @@ __device__ __forceinline__ void ce_emit(float (&g)[VecOf<T>::N], int vi, int mis
     }
 }
 
+// Issues the asynchronous copies of row `xr_` (cols elements) into the landing area:
+// thread t owns slots t, t + CE_THREADS, ...; threads past the row re-read its last vector.
+template <typename T, int ITERS>
+__device__ __forceinline__ void ce_issue_row(const T* xr_, int cols, int t, char* land) {
+    constexpr int VEC = VecOf<T>::N;
+    const int mis_ = (int)((reinterpret_cast<uintptr_t>(xr_) & 15) / sizeof(T));
+    const T* xb_ = xr_ - mis_;
+    const int nvec_ = (cols + mis_ + VEC - 1) / VEC;
+    const char* gb = reinterpret_cast<const char*>(xb_);
+    // a rolled loop on purpose: unrolled, the eight 64-bit addresses are hoisted out of the
+    // row loop and spilled
+#pragma unroll 1
+    for (int it = 0; it < ITERS; ++it) {
+        const int vi = t + it * CE_THREADS;
+        const uint32_t vc = (uint32_t)(vi < nvec_ ? vi : nvec_ - 1);
+        ce_load_to_lds(gb + vc * 16u, land + ((t & ~63) + it * CE_THREADS) * 16);
+    }
+}
+
 // CACHED: the row is kept in registers (ITERS vectors per thread).  Otherwise the
 // row is streamed from memory three times (max, sum, gradient).
 template <typename T, int ITERS, bool CACHED>
@@ -57,12 +85,21 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                                                        const int64_t* __restrict__ count, int64_t rows, int cols,
                                                        int64_t xs, int64_t dxs) {
     constexpr int VEC = VecOf<T>::N;
+    // 2-byte rows are fetched with asynchronous global->LDS copies: every vector of the row
+    // is in flight at once at no register cost, a thread reads back only the slots it
+    // filled itself (no barrier), and the next row's copies are issued as soon as this
+    // row sits in registers, so they overlap the reductions and the gradient stores.
+    constexpr bool LAND = CACHED && sizeof(T) == 2;
+    __shared__ __attribute__((aligned(16))) char land[LAND ? CE_THREADS * ITERS * 16 : 16];
     __shared__ float smem[16];
     __shared__ int smin[16];
     __shared__ float s_xy;
-    const int t = threadIdx.x;
     const float inv_cnt = 1.0f / (float)(*count);
+    if constexpr (LAND) {
+        if ((int64_t)blockIdx.x < rows) ce_issue_row<T, ITERS>(logits + (int64_t)blockIdx.x * xs, cols, threadIdx.x, land);
+    }
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const int t = threadIdx.x;
         const T* xr = logits + row * xs;
         T* dr = dlogits + row * dxs;
         const int mis = (int)((reinterpret_cast<uintptr_t>(xr) & 15) / sizeof(T));
@@ -74,7 +111,29 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
 
         float v[ITERS][VEC];
         float m = -INFINITY;
-        if constexpr (CACHED) {
+        if constexpr (LAND) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this row's copies have landed
+            // thread index behind an opaque barrier: the slot offsets are recomputed here
+            // instead of being hoisted out of the row loop and spilled
+            int tr = t;
+            asm volatile("" : "+v"(tr));
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int vi = tr + it * CE_THREADS;
+                const ce_u32x4 raw = *reinterpret_cast<const ce_u32x4*>(land + vi * 16);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int e = vi * VEC + j - mis;
+                    const float x = __uint_as_float((j & 1) ? (raw[j >> 1] & 0xffff0000u) : (raw[j >> 1] << 16));
+                    v[it][j] = (e < 0 || e >= cols) ? -INFINITY : x;
+                    m = fmaxf(m, v[it][j]);
+                }
+                // two LDS reads in flight are enough; more would only cost registers
+                if (it & 1) __builtin_amdgcn_sched_barrier(0);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // slots are free again
+            if (row + gridDim.x < rows) ce_issue_row<T, ITERS>(logits + (row + gridDim.x) * xs, cols, t, land);
+        } else if constexpr (CACHED) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int vi = t + it * CE_THREADS;
@@ -164,9 +223,11 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
         const float scale = live ? inv_cnt / s : 0.f;
 
         if constexpr (CACHED) {
+            int ts = t;
+            asm volatile("" : "+v"(ts));   // as above: keep the store offsets out of the spill area
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
-                const int vi = t + it * CE_THREADS;
+                const int vi = ts + it * CE_THREADS;
                 if (vi < nvec) {
                     float g[VEC];
 #pragma unroll
