@@ -19,8 +19,8 @@
 //
 // Dropout on the probabilities: element (q, k) of batch-head g is kept iff
 // philox(seed + g, q + k) passes the threshold -- the offset depends on q + k only, so
-// one line of 2T keep bits per batch-head is generated once (attn_keepbits_kernel) and
-// every kernel extracts a lane's 32-key window from it with one 64-bit shift.
+// one line of 2T keep bits per batch-head is generated once (attn_keepbits_kernel); the
+// kernels read it through the scalar unit and turn it into 64-lane select masks.
 //
 // The backward is two passes without atomics: (dK, dV) over key tiles, dQ over query
 // tiles; both recompute S and dP.
@@ -140,11 +140,53 @@ __device__ __forceinline__ void tp_x_regs(f32x16 (&o)[2], const char* __restrict
     for (int j = 0; j < 2; ++j) tp_x_regs_one(o, panels, p[j], j, lr, lg, tag);
 }
 
-// 32 keep bits starting at bit `ob` of the batch-head's bit line (LDS copy).
-__device__ __forceinline__ uint32_t keep_window(const uint32_t* __restrict__ sbits, int ob) {
-    const int w = ob >> 5, sh = ob & 31;
-    const uint64_t v = ((uint64_t)sbits[w + 1] << 32) | sbits[w];
-    return (uint32_t)(v >> sh);
+// Keep bits of one wavefront tile as wave-uniform (scalar) words.  Element (q, k) is kept
+// iff bit q + k of the batch-head's line is set.  In the kernels whose lanes are queries
+// (keys), the element in accumulator register i of sub-tile j sits at
+//   q + k = base + C + (lane & 31) + 4 * (lane >> 5),   C = 32 j + 8 (i / 4) + i % 4,
+// with base = (wave's first query) + (tile's first key), a multiple of 32.  So the keep
+// decision of ONE register across the 64 lanes is two 32-bit windows of the line at the
+// constant offsets C and C + 4: a lane mask that the scalar unit extracts with two
+// shifts and that a single v_cndmask applies -- no per-lane bit arithmetic at all.
+struct KeepWords { uint32_t d0, d1, d2; };
+__device__ __forceinline__ KeepWords load_keep_words(const uint32_t* __restrict__ line, int base) {
+    const uint32_t* p = line + (base >> 5);   // wave-uniform address: scalar loads
+    KeepWords w;
+    w.d0 = p[0];
+    w.d1 = p[1];
+    w.d2 = p[2];
+    return w;
+}
+template <int C> __device__ __forceinline__ uint32_t keep_win32(const KeepWords& w) {
+    static_assert(C >= 0 && C < 64, "window offset");
+    const uint64_t v = C < 32 ? (((uint64_t)w.d1 << 32) | w.d0) : (((uint64_t)w.d2 << 32) | w.d1);
+    return (uint32_t)(v >> (C & 31));
+}
+template <int C> __device__ __forceinline__ uint64_t keep_lane_mask(const KeepWords& w) {
+    return (uint64_t)keep_win32<C>(w) | ((uint64_t)keep_win32<C + 4>(w) << 32);
+}
+// v where the lane's bit of `mask` is set, else 0.  The builtin turns a wave-uniform 64-bit
+// mask into a per-lane condition, i.e. one v_cndmask with the mask in scalar registers
+// (left to the compiler rather than inline assembly so that its hazard handling --
+// e.g. the wait state after a transcendental -- still applies).
+__device__ __forceinline__ float keep_select(float v, uint64_t mask) {
+    return __builtin_amdgcn_inverse_ballot_w64(mask) ? v : 0.f;
+}
+// the 16 lane masks of sub-tile J
+template <int J, int I = 0>
+__device__ __forceinline__ void keep_masks(uint64_t (&m)[16], const KeepWords& w) {
+    if constexpr (I < 16) {
+        m[I] = keep_lane_mask<J * 32 + (I >> 2) * 8 + (I & 3)>(w);
+        keep_masks<J, I + 1>(m, w);
+    }
+}
+// p[i] = keep ? p[i] : 0 for the 16 registers of sub-tile J
+template <int J, int I = 0>
+__device__ __forceinline__ void keep_apply(float (&p)[16], const KeepWords& w) {
+    if constexpr (I < 16) {
+        p[I] = keep_select(p[I], keep_lane_mask<J * 32 + (I >> 2) * 8 + (I & 3)>(w));
+        keep_apply<J, I + 1>(p, w);
+    }
 }
 
 // Store the transposed accumulators acc[t][i] (row = the lane's position `pos`, column
@@ -242,7 +284,6 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
     typedef AT<T> X;
     constexpr int STAGE = 2 * X::NP * PANEL;  // K panels then V^T panels
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
-    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -281,10 +322,9 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
     }
 
     FWD_FETCH(0)
-    if constexpr (TRAIN) {
-        const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
-        for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
-    }
+    // keep-bit line of this batch-head and the wave's first query as scalars
+    const uint32_t* __restrict__ kline = a.keepbits + (int64_t)bh * a.bitwords;
+    const int qw0u = q0 + __builtin_amdgcn_readfirstlane(wave) * 32;
     FWD_STASH(0)
     __syncthreads();
 
@@ -296,9 +336,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
 
+    KeepWords kw_next;
+    if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u);
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
         FWD_FETCH(kt + 1 < nkt ? kt + 1 : kt)
+        // keep bits of this tile were requested one step ago; request the next tile's now
+        const KeepWords kw = kw_next;
+        if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u + (kt + 1) * 64);
         __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {   // some key of this tile is visible to some query of the wave
@@ -354,12 +399,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
 #pragma unroll
                 for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
             if constexpr (TRAIN) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) p[j][i] = and_bits(p[j][i], bit_mask(w, (i >> 2) * 8 + (i & 3)));
-                }
+                keep_apply<0>(p[0], kw);
+                keep_apply<1>(p[1], kw);
             }
             tp_x_regs(o, vp, p, lr, lg, T());
         }
@@ -388,7 +429,6 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     constexpr int STAGE = 4 * X::NP * PANEL;  // Q, dO, Q^T, dO^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
     __shared__ __attribute__((aligned(16))) float sstat[2][3][64];  // m2, 1/l, delta per stage
-    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -450,18 +490,21 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 
     if (qt0 < nqt) {
         KV_FETCH(qt0)
-        if constexpr (TRAIN) {
-            const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
-            for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
-        }
         KV_STASH(0)
     }
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
+    // keep-bit line of this batch-head and the wave's first key as scalars
+    const uint32_t* __restrict__ kline = a.keepbits + (int64_t)bh * a.bitwords;
+    const int kw0u = key0 + __builtin_amdgcn_readfirstlane(wave) * 32;
+    KeepWords kw_next;
+    if constexpr (TRAIN) kw_next = load_keep_words(kline, kw0u + qt0 * 64);
     for (int qt = qt0; qt < nqt; ++qt) {
         const int st = (qt - qt0) & 1;
         KV_FETCH(qt + 1 < nqt ? qt + 1 : qt)
+        const KeepWords kw = kw_next;   // requested one step ago
+        if constexpr (TRAIN) kw_next = load_keep_words(kline, kw0u + (qt + 1) * 64);
         __builtin_amdgcn_sched_barrier(0);
         const int q0 = qt * 64;
         if (q0 + 63 >= kw0) {   // some query of the tile sees some key of the wave
@@ -490,8 +533,11 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                     }
                 }
                 float pd[16], ds[16];
-                uint32_t w = 0;
-                if constexpr (TRAIN) w = keep_window(sbits, key + q0 + j * 32 + lg * 4);
+                uint64_t km[16];
+                if constexpr (TRAIN) {
+                    if (j == 0) keep_masks<0>(km, kw);
+                    else keep_masks<1>(km, kw);
+                }
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const int qi = j * 32 + g4 * 8 + lg * 4;  // first of 4 consecutive queries (tile-relative)
@@ -503,9 +549,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                         const int i = g4 * 4 + b;
                         const float p = fast_exp2(fmaf(s[i], sc, -m4[b])) * l4[b];
                         if constexpr (TRAIN) {
-                            const int32_t km = bit_mask(w, g4 * 8 + b);
-                            pd[i] = and_bits(p, km);
-                            ds[i] = p * (and_bits(dp[i], km) - d4[b]);
+                            pd[i] = keep_select(p, km[i]);
+                            ds[i] = p * (keep_select(dp[i], km[i]) - d4[b]);
                         } else {
                             pd[i] = 0.9f * p;
                             ds[i] = p * fmaf(dp[i], 0.9f, -d4[b]);
@@ -540,7 +585,6 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     typedef AT<T> X;
     constexpr int STAGE = 3 * X::NP * PANEL;  // K, V, K^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
-    __shared__ uint32_t sbits[TRAIN ? MAX_BITWORDS : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lg = lane >> 5;
@@ -580,10 +624,6 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     }
 
     DQ_FETCH(0)
-    if constexpr (TRAIN) {
-        const uint32_t* gb = a.keepbits + (int64_t)bh * a.bitwords;
-        for (int i = tid; i < a.bitwords; i += ATT_THREADS) sbits[i] = gb[i];
-    }
     DQ_STASH(0)
     __syncthreads();
 
@@ -594,9 +634,15 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 #pragma unroll
         for (int e = 0; e < 16; ++e) dq[t][e] = 0.f;
 
+    const uint32_t* __restrict__ kline = a.keepbits + (int64_t)bh * a.bitwords;
+    const int qw0u = q0 + __builtin_amdgcn_readfirstlane(wave) * 32;
+    KeepWords kw_next;
+    if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u);
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
         DQ_FETCH(kt + 1 < nkt ? kt + 1 : kt)
+        const KeepWords kw = kw_next;   // requested one step ago
+        if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u + (kt + 1) * 64);
         __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {
@@ -634,13 +680,16 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
             float ds[2][16];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t w = 0;
-                if constexpr (TRAIN) w = keep_window(sbits, query + key0 + j * 32 + lg * 4);
+                uint64_t km[16];
+                if constexpr (TRAIN) {
+                    if (j == 0) keep_masks<0>(km, kw);
+                    else keep_masks<1>(km, kw);
+                }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const float p = fast_exp2(fmaf(s[j][i], sc, -m2)) * linv;
                     if constexpr (TRAIN)
-                        ds[j][i] = p * (and_bits(dp[j][i], bit_mask(w, (i >> 2) * 8 + (i & 3))) - delta);
+                        ds[j][i] = p * (keep_select(dp[j][i], km[i]) - delta);
                     else
                         ds[j][i] = p * fmaf(dp[j][i], 0.9f, -delta);
                 }
