@@ -152,6 +152,16 @@ int ptj_adamw(float* p, float* m, float* v, const void* g, void* shadow, int64_t
               float lr, float beta1, float beta2, float eps, float weight_decay, int64_t t,
               int grad_dtype, int shadow_dtype, void* stream);
 
+/* The same update for `count` tensors in as few launches as possible (the whole
+ * parameter nest of adam_w_in_place, loss_and_optimizer_triton.py:376-401, in one call).
+ * p, m, v, g, shadow, n and weight_decay are HOST arrays of `count` entries (shadow may be
+ * NULL: no low-precision copies); all gradients share grad_dtype and all shadows
+ * shadow_dtype.  Each tensor is updated exactly as by ptj_adamw. */
+int ptj_adamw_multi(int64_t count, float* const* p, float* const* m, float* const* v,
+                    const void* const* g, void* const* shadow, const int64_t* n,
+                    const float* weight_decay, float lr, float beta1, float beta2, float eps,
+                    int64_t t, int grad_dtype, int shadow_dtype, void* stream);
+
 /* ---- attention ----------------------------------------------------------- */
 
 /* Causal flash-attention forward.  q/k/v/o are [B, H, T, dh] views with explicit

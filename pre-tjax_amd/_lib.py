@@ -39,6 +39,8 @@ SIGNATURES = {
                         _p]),
     "ptj_adamw": (_int, [_p, _p, _p, _p, _p, _i64, _c.c_float, _c.c_float, _c.c_float, _c.c_float, _c.c_float, _i64,
                          _int, _int, _p]),
+    "ptj_adamw_multi": (_int, [_i64, _p, _p, _p, _p, _p, _p, _p, _c.c_float, _c.c_float, _c.c_float, _c.c_float, _i64,
+                               _int, _int, _p]),
     "ptj_attn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ptj_attn_fwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz] + [_i64] * 16 + [_int, _i64, _int, _p]),
     "ptj_attn_bwd": (_int, [_p] * 11 + [_p, _sz] + [_i64] * 28 + [_int, _i64, _int, _p]),

@@ -1,5 +1,7 @@
 """Loss-side wrappers with the reference's names (loss_and_optimizer_triton.py of
 martin-kukla/pre-tjax) on top of libptj.so."""
+import ctypes
+
 import torch
 
 from ._lib import check, dtype_code, lib, ptr, require_gpu, stream
@@ -74,20 +76,38 @@ def init_adam_w(params):
 def adam_w_in_place(master, grads, lr, betas, epsilon, moments, i, weight_decay=0.0, weight_decay_mask=None,
                     shadow=None):
     """AdamW of the reference (:376-401: t = i+1, bias-corrected moments, decay scaled by
-    lr) on fp32 master weights: one fused HIP pass per tensor instead of ~10 torch ops.
+    lr) on fp32 master weights: one fused HIP pass over the whole nest (a few launches)
+    instead of ~10 torch ops per tensor.
     `shadow` (optional nest of low-precision copies) is refreshed from the masters."""
     t = i + 1
-    st = stream()
-    fn = lib().ptj_adamw
+    ps, ms_, vs, gs, ss, ns, wds = [], [], [], [], [], [], []
+    keep = []                                    # contiguous gradient copies must outlive the launch
+    gdt = sdt = None
     for gi, grp in enumerate(master):
         for pi, p in enumerate(grp):
             g = grads[gi][pi]
             if not g.is_contiguous():
                 g = g.contiguous()
-            wd = weight_decay if (weight_decay_mask is None or weight_decay_mask[gi][pi]) else 0.0
+                keep.append(g)
             sh = shadow[gi][pi] if shadow is not None else None
             assert p.dtype == torch.float32 and p.is_contiguous() and g.numel() == p.numel()
-            check(fn(ptr(p), ptr(moments[0][gi][pi]), ptr(moments[1][gi][pi]), ptr(g), ptr(sh), p.numel(), lr,
-                     betas[0], betas[1], epsilon, wd, t, dtype_code(g), dtype_code(sh) if sh is not None else -1, st),
-                  "ptj_adamw")
+            assert gdt in (None, g.dtype) and (sh is None or sdt in (None, sh.dtype)), "mixed gradient / shadow dtypes"
+            gdt = g.dtype
+            if sh is not None:
+                sdt = sh.dtype
+            ps.append(p.data_ptr())
+            ms_.append(moments[0][gi][pi].data_ptr())
+            vs.append(moments[1][gi][pi].data_ptr())
+            gs.append(g.data_ptr())
+            ss.append(sh.data_ptr() if sh is not None else 0)
+            ns.append(p.numel())
+            wds.append(weight_decay if (weight_decay_mask is None or weight_decay_mask[gi][pi]) else 0.0)
+    cnt = len(ps)
+    if cnt:
+        arr = lambda vals: (ctypes.c_void_p * cnt)(*vals)
+        code = {torch.float32: 0, torch.bfloat16: 1}
+        check(lib().ptj_adamw_multi(cnt, arr(ps), arr(ms_), arr(vs), arr(gs), arr(ss) if shadow is not None else None,
+                                    (ctypes.c_int64 * cnt)(*ns), (ctypes.c_float * cnt)(*wds), lr, betas[0], betas[1],
+                                    epsilon, t, code[gdt], code[sdt] if sdt is not None else -1, stream()),
+              "ptj_adamw_multi")
     return master, moments
