@@ -64,6 +64,21 @@ int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const vo
                       int64_t rows, int64_t cols, int64_t dy_row_stride, int64_t x_row_stride,
                       int64_t dx_row_stride, int dtype, void* stream);
 
+/* ptj_layernorm_bwd with a second output: `dropped` (nullable, contiguous [rows, cols]) =
+ * dropout(dx) computed from the stored dx with the mask of ptj_dropout(train, seed) --
+ * the t_dropout_bkwd2_t that the block backward applies to every residual-stream gradient
+ * (model_triton.py:2021-2024, 2175-2178) without another pass over dx.  Bit-identical to
+ * ptj_layernorm_bwd followed by ptj_dropout.  `keep_bytes` (nullable) are the keep bits
+ * that ptj_dropout_add_keep recorded for the same (seed, shape); with them the mask is
+ * read instead of recomputed (2-byte element types only). */
+int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, const void* residual,
+                              void* dx, void* dgamma, void* dbeta,
+                              void* dropped, int drop_train, int64_t drop_seed,
+                              const void* keep_bytes,
+                              void* workspace, size_t workspace_bytes,
+                              int64_t rows, int64_t cols, int64_t dy_row_stride, int64_t x_row_stride,
+                              int64_t dx_row_stride, int dtype, void* stream);
+
 /* Column sums out[c] = sum_r x[r, c] (bias gradients: the `.sum(dim=0)` of
  * t_linear_bkwd2_p, model_triton.py:426).  Two-stage, fixed order.  `workspace`:
  * ptj_colsum_workspace_bytes(rows, cols) bytes. */
@@ -89,6 +104,13 @@ int ptj_dropout(const void* x, void* y, int64_t rows, int64_t cols,
  * All three tensors are contiguous [rows, cols]. */
 int ptj_dropout_add(const void* x, const void* res, void* y, int64_t rows, int64_t cols,
                     int train, int64_t seed, int dtype, void* stream);
+
+/* ptj_dropout_add that also records its keep mask: keep_bytes[r * cols/8 + g] holds, in
+ * bit j, whether column 8g + j of row r was kept (train != 0).  The backward
+ * (ptj_layernorm_bwd_dropout) can then read the mask instead of re-running Philox.
+ * Needs a 2-byte element type, cols % 8 == 0 and 16-byte aligned tensors. */
+int ptj_dropout_add_keep(const void* x, const void* res, void* y, void* keep_bytes,
+                         int64_t rows, int64_t cols, int train, int64_t seed, int dtype, void* stream);
 
 /* Row-wise log-softmax forward / backward (dx = dy - softmax(x)*sum(dy)).
  * Replace t_log_softmax_fwd_k/_t (model_triton.py:30-72) and

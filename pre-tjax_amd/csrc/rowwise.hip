@@ -102,7 +102,8 @@ constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave ho
 template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
 __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
-    T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs) {
+    T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs,
+    T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep) {
     __shared__ float smem[16];
     constexpr int RPB = LnBwdGeom<TPR>::ROWS_PER_BLOCK;
     const int t = threadIdx.x % TPR;
@@ -184,6 +185,32 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                     for (int j = 0; j < VEC; ++j) d.v[it][j] = rr.v[it][j] + to_f32(from_f32<T>(d.v[it][j]));
             }
             d.store(dx + row * dxs, nvec, t);
+            if (drop != nullptr) {
+                // second output: dropout applied to the stored (rounded) dx, i.e. the backward
+                // of the dropout that feeds this residual stream -- saves a pass over dx
+                const uint64_t sd = drop_seed + (uint64_t)row;
+                const uint32_t k0 = (uint32_t)sd, k1 = (uint32_t)(sd >> 32);
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it) {
+                    const int vi = t + it * TPR;
+                    // keep bits of this vector: recorded by the forward dropout (one byte per
+                    // 8 columns) when available, else recomputed
+                    uint32_t bits = 0;
+                    if (VEC == 8 && keep != nullptr) {
+                        bits = keep[row * (int64_t)nvec + (vi < nvec ? vi : nvec - 1)];
+                    } else if (drop_train) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j)
+                            bits |= philox_keep((uint32_t)(vi * VEC + j), k0, k1) ? (1u << j) : 0u;
+                    }
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const float r = to_f32(from_f32<T>(d.v[it][j]));
+                        d.v[it][j] = drop_train ? (((bits >> j) & 1u) ? r : 0.f) : r * 0.9f;
+                    }
+                }
+                d.store(drop + row * (int64_t)cols, nvec, t);
+            }
         }
     }
     if constexpr (DGB) {
@@ -378,7 +405,8 @@ __global__ __launch_bounds__(256) void gelu_bwd_kernel(const T* __restrict__ dy,
 template <typename T, int VEC, bool ADD>
 __global__ __launch_bounds__(256) void dropout_kernel(const T* __restrict__ x, const T* __restrict__ res,
                                                        T* __restrict__ y, int64_t rows, int cols, int64_t xs,
-                                                       int64_t ys, int train, uint64_t seed) {
+                                                       int64_t ys, int train, uint64_t seed,
+                                                       uint8_t* __restrict__ keep_out) {
     const int vpr = cols / VEC;  // vectors per row
     const int64_t total = rows * vpr;
     const bool small = total <= 0x7fffffffll;  // 32-bit division is several times cheaper
@@ -390,8 +418,15 @@ __global__ __launch_bounds__(256) void dropout_kernel(const T* __restrict__ x, c
         if (train) {
             const uint64_t s = seed + (uint64_t)row;
             const uint32_t k0 = (uint32_t)s, k1 = (uint32_t)(s >> 32);
+            uint32_t bits = 0;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] = philox_keep((uint32_t)(c0 + j), k0, k1) ? v[j] : 0.f;
+            for (int j = 0; j < VEC; ++j) {
+                const bool keep = philox_keep((uint32_t)(c0 + j), k0, k1);
+                v[j] = keep ? v[j] : 0.f;
+                bits |= keep ? (1u << j) : 0u;
+            }
+            // keep byte of this 8-column group (only requested on the 8-wide path)
+            if (VEC == 8 && keep_out != nullptr) keep_out[i] = (uint8_t)bits;
         } else {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= 0.9f;
@@ -579,9 +614,11 @@ template <typename T>
 int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const void* res, void* dx, void* dgamma,
                        void* dbeta,
                        void* ws, size_t ws_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs, int64_t dxs,
-                       hipStream_t st) {
+                       void* drop, int drop_train, int64_t drop_seed, const void* keep, hipStream_t st) {
     RowCfg cfg;
-    const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx, res}, {dys, xs, dx ? dxs : 0});
+    const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx, res, drop}, {dys, xs, dx ? dxs : 0});
+    if (keep != nullptr && !(vok && VecOf<T>::N == 8))
+        return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: keep bytes need 2-byte elements and the vector path");
     if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
         return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: cols=%lld too large", (long long)cols);
     const int grid = ln_bwd_grid(rows, cfg.tpr);
@@ -595,7 +632,8 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
 #define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_)                                                                   \
     hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
                        dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (const T_*)res, (T_*)dx, \
-                       (float*)ws, rows, (int)cols, dys, xs, dxs)
+                       (float*)ws, rows, (int)cols, dys, xs, dxs, (T_*)drop, drop_train, (uint64_t)drop_seed,    \
+                       (const uint8_t*)keep)
 #define LAUNCH(T_, V_, TPR_, IT_)                                     \
     do {                                                              \
         if (want_dx && want_dgb) LAUNCH_F(T_, V_, TPR_, IT_, true, true);   \
@@ -681,14 +719,17 @@ int gelu_impl(const void* dy, const void* x, void* out, int64_t n, bool bwd, hip
 
 template <typename T>
 int dropout_impl(const void* x, const void* res, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
-                 int train, int64_t seed, hipStream_t st) {
+                 int train, int64_t seed, hipStream_t st, void* keep_out = nullptr) {
     constexpr int FV = VecOf<T>::N;
     if (rows == 0 || cols == 0) return PTJ_OK;
     const bool vok = (cols % FV == 0) && (xs % FV == 0) && (ys % FV == 0) && ptj_aligned16(x) && ptj_aligned16(y) &&
                      (!res || ptj_aligned16(res));
+    if (keep_out != nullptr && !(vok && FV == 8))
+        return ptj_set_error(PTJ_ERR_INVALID, "dropout: keep bytes need 2-byte elements, cols %% 8 == 0 and 16-byte aligned rows");
 #define LAUNCH(V_, ADD_)                                                                                       \
     hipLaunchKernelGGL((dropout_kernel<T, V_, ADD_>), dim3(flat_grid(rows * (cols / V_))), dim3(256), 0, st,     \
-                       (const T*)x, (const T*)res, (T*)y, rows, (int)cols, xs, ys, train, (uint64_t)seed)
+                       (const T*)x, (const T*)res, (T*)y, rows, (int)cols, xs, ys, train, (uint64_t)seed,       \
+                       (uint8_t*)keep_out)
     if (vok) {
         if (res) LAUNCH(FV, true); else LAUNCH(FV, false);
     } else {
@@ -728,23 +769,32 @@ size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
     return (size_t)512 * 2 * (size_t)cols * sizeof(float);
 }
 
-int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const void* residual, void* dx, void* dgamma,
-                      void* dbeta,
-                      void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
-                      int64_t dxs, int dtype, void* stream) {
+int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, const void* residual, void* dx,
+                              void* dgamma, void* dbeta, void* dropped, int drop_train, int64_t drop_seed,
+                              const void* keep_bytes, void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys,
+                              int64_t xs, int64_t dxs, int dtype, void* stream) {
     PTJ_CHECK_ARG(dy && x, "layernorm_bwd: null dy/x");
     PTJ_CHECK_ARG(dx || dgamma, "layernorm_bwd: nothing to compute (dx and dgamma both null)");
     PTJ_CHECK_ARG(!dx || gamma, "layernorm_bwd: dx requested without gamma");
     PTJ_CHECK_ARG(!residual || dx, "layernorm_bwd: residual given without dx");
+    PTJ_CHECK_ARG(!dropped || dx, "layernorm_bwd: dropout output requested without dx");
     PTJ_CHECK_ARG((dgamma == nullptr) == (dbeta == nullptr), "layernorm_bwd: dgamma and dbeta must be given together");
     PTJ_CHECK_ARG(rows >= 1 && cols >= 2, "layernorm_bwd: need rows >= 1 and cols >= 2");
     PTJ_CHECK_ARG(dys >= cols && xs >= cols && (!dx || dxs >= cols), "layernorm_bwd: row stride smaller than cols");
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype,
                  (layernorm_bwd_impl<float>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols,
-                                            dys, xs, dxs, st)),
+                                            dys, xs, dxs, dropped, drop_train, drop_seed, keep_bytes, st)),
                  (layernorm_bwd_impl<bf16>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols, dys,
-                                           xs, dxs, st)));
+                                           xs, dxs, dropped, drop_train, drop_seed, keep_bytes, st)));
+}
+
+int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const void* residual, void* dx, void* dgamma,
+                      void* dbeta,
+                      void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
+                      int64_t dxs, int dtype, void* stream) {
+    return ptj_layernorm_bwd_dropout(dy, x, gamma, residual, dx, dgamma, dbeta, nullptr, 0, 0, nullptr, workspace, workspace_bytes,
+                                     rows, cols, dys, xs, dxs, dtype, stream);
 }
 
 size_t ptj_colsum_workspace_bytes(int64_t rows, int64_t cols) {
@@ -801,6 +851,16 @@ int ptj_dropout_add(const void* x, const void* res, void* y, int64_t rows, int64
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype, (dropout_impl<float>(x, res, y, rows, cols, cols, cols, train, seed, st)),
                  (dropout_impl<bf16>(x, res, y, rows, cols, cols, cols, train, seed, st)));
+}
+
+int ptj_dropout_add_keep(const void* x, const void* res, void* y, void* keep_bytes, int64_t rows, int64_t cols,
+                         int train, int64_t seed, int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 0, "dropout_add_keep: negative shape");
+    PTJ_CHECK_ARG(rows * cols == 0 || (x && res && y && keep_bytes), "dropout_add_keep: null pointer");
+    PTJ_CHECK_ARG(cols < (1ll << 31), "dropout_add_keep: cols must fit in 31 bits");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (dropout_impl<float>(x, res, y, rows, cols, cols, cols, train, seed, st, keep_bytes)),
+                 (dropout_impl<bf16>(x, res, y, rows, cols, cols, cols, train, seed, st, keep_bytes)));
 }
 
 int ptj_log_softmax_fwd(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, int dtype,

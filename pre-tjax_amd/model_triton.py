@@ -107,9 +107,17 @@ def t_dropout_bkwd2_t(dloss_dx: torch.Tensor, x: torch.Tensor, train=True, p_gen
     return _dropout(dloss_dx, train, p_gen_aux)
 
 
-def dropout_add_t(x: torch.Tensor, residual: torch.Tensor, train=True, p_gen_aux=None):
+def _keep_bytes_ok(t):
+    """Keep bytes (one per 8 columns) exist for 2-byte element types with 8-column rows."""
+    return t.element_size() == 2 and t.shape[-1] % 8 == 0 and t.data_ptr() % 16 == 0
+
+
+def dropout_add_t(x: torch.Tensor, residual: torch.Tensor, train=True, p_gen_aux=None, want_keep=False):
     """residual + dropout(x) in one pass (the `y + t_dropout_fwd_t(y_diff, ...)` of
-    model_triton.py:1898 and :2069)."""
+    model_triton.py:1898 and :2069).  With ``want_keep`` the result is (out, keep) where
+    `keep` holds the keep mask as one byte per 8 columns (None when the mask is not
+    recorded: eval mode, or a layout without keep bytes); the backward reads it instead
+    of recomputing the Philox stream."""
     require_gpu(x, residual)
     assert x.shape == residual.shape and x.dtype == residual.dtype
     if not train:
@@ -118,9 +126,14 @@ def dropout_add_t(x: torch.Tensor, residual: torch.Tensor, train=True, p_gen_aux
     out = torch.empty_like(xc)
     cols = xc.shape[-1]
     rows = xc.numel() // cols
+    if want_keep and train and _keep_bytes_ok(xc) and _keep_bytes_ok(rc):
+        keep = torch.empty(rows * (cols // 8), dtype=torch.uint8, device=xc.device)
+        check(lib().ptj_dropout_add_keep(ptr(xc), ptr(rc), ptr(out), ptr(keep), rows, cols, 1, int(p_gen_aux),
+                                         dtype_code(xc), stream()), "ptj_dropout_add_keep")
+        return out, keep
     check(lib().ptj_dropout_add(ptr(xc), ptr(rc), ptr(out), rows, cols, int(bool(train)), int(p_gen_aux),
                                 dtype_code(xc), stream()), "ptj_dropout_add")
-    return out
+    return (out, None) if want_keep else out
 
 
 # ----------------------------------------------------------------------------------
@@ -138,7 +151,7 @@ def t_layernorm_fwd_t(layer_params, x: torch.Tensor):
     return out.reshape(x.shape)
 
 
-def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None):
+def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None, drop=None):
     require_gpu(dloss_dx, x)
     d2, x2 = _rows2d(dloss_dx), _rows2d(x)
     assert d2.shape == x2.shape and d2.dtype == x2.dtype
@@ -154,10 +167,21 @@ def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None):
     if residual is not None:
         assert want_dx and residual.shape == x.shape and residual.dtype == x2.dtype
         residual = residual.contiguous()
-    check(lib().ptj_layernorm_bwd(ptr(d2), ptr(x2), ptr(gamma), ptr(residual), ptr(dx), ptr(dg), ptr(db), ptr(ws), ws_bytes,
-                                  rows, cols, d2.stride(0), x2.stride(0), dx.stride(0) if want_dx else 0,
-                                  dtype_code(x2), stream()), "ptj_layernorm_bwd")
-    return (dx.reshape(dloss_dx.shape) if want_dx else None), dg, db
+    dropped, d_train, d_seed = None, 0, 0
+    keep = None
+    if drop is not None:                         # (train, seed[, keep bytes]): also emit dropout_bkwd(dx)
+        assert want_dx
+        d_train, d_seed = int(bool(drop[0])), int(drop[1] if drop[0] else 0)
+        keep = drop[2] if len(drop) > 2 and drop[0] else None
+        dropped = torch.empty_like(dx)
+    check(lib().ptj_layernorm_bwd_dropout(ptr(d2), ptr(x2), ptr(gamma), ptr(residual), ptr(dx), ptr(dg), ptr(db),
+                                          ptr(dropped), d_train, d_seed, ptr(keep), ptr(ws), ws_bytes, rows, cols, d2.stride(0),
+                                          x2.stride(0), dx.stride(0) if want_dx else 0, dtype_code(x2), stream()),
+          "ptj_layernorm_bwd")
+    dx_out = dx.reshape(dloss_dx.shape) if want_dx else None
+    if drop is not None:
+        return dx_out, dg, db, dropped.reshape(dloss_dx.shape)
+    return dx_out, dg, db
 
 
 def t_layernorm_bkwd2_p_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor):
@@ -170,9 +194,15 @@ def t_layernorm_bkwd2_x_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor)
     return dx
 
 
-def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, residual=None):
+def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, residual=None, drop=None):
     """dx (+ residual), (dgamma, dbeta) from one read of dy and x (fusion of the two
-    reference launches at model_triton.py:2033-2034 and of the residual add at :2036)."""
+    reference launches at model_triton.py:2033-2034 and of the residual add at :2036).
+    With ``drop=(train, seed[, keep])`` a third result is t_dropout_bkwd2_t(dx, None, train,
+    seed) (the dropout backward the block applies next, :2021-2024), written in the same
+    pass; `keep` are the keep bytes recorded by dropout_add_t for that seed, if any."""
+    if drop is not None:
+        dx, dg, db, dropped = _layernorm_bwd(dloss_dx, layer_params, x, True, True, residual, drop)
+        return dx, (dg, db), dropped
     dx, dg, db = _layernorm_bwd(dloss_dx, layer_params, x, True, True, residual)
     return dx, (dg, db)
 
@@ -398,29 +428,34 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
     o4 = o2.view(B, T, H, dh).permute(0, 2, 1, 3)
     _, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux[0], out=o4)
     a_out = matmul_t(o2, wo.t())
-    x_mid = dropout_add_t(a_out, x_in, train, p_gen_aux[1])
+    x_mid, keep1 = dropout_add_t(a_out, x_in, train, p_gen_aux[1], want_keep=True)
     h2 = t_layernorm_fwd_t((ln2g, ln2b), x_mid)
     f1 = torch.empty((N, w1.shape[0]), dtype=y.dtype, device=y.device)
     g1 = matmul_t(h2, w1.t(), b1, gelu=True, pre_out=f1)               # bias + GELU epilogue, both kept
     f2 = matmul_t(g1, w2.t(), b2)
-    x_out = dropout_add_t(f2, x_mid, train, p_gen_aux[2])
-    acts = (x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1)
+    x_out, keep2 = dropout_add_t(f2, x_mid, train, p_gen_aux[2], want_keep=True)
+    acts = (x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1, keep1, keep2)
     return x_out.view(B, T, D), acts
 
 
-def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_aux=None):
+def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_aux=None, dropped_in=None,
+                          drop_out=None):
     """Backward of one block (model_triton.py:2291-2299 and the sub-block VJPs :2021-2039,
-    :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order)."""
+    :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order).
+
+    `dropped_in`, if given, is t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2]) already
+    computed by the producer of dloss_dx; `drop_out=(train, seed)` asks for the same service
+    for the consumer of dx: the result is then (dx, grads, dropout_bkwd(dx))."""
     if not train:
         p_gen_aux = [0, 0, 0]
     ln1g, ln1b, wqkv, wo, ln2g, ln2b, w1, b1, w2, b2 = layer_params
-    x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1 = acts
+    x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1, keep1, _ = acts
     H, _, dh, D = wqkv.shape
     N = x_in.shape[0]
     T = ms.shape[2]
     B = N // T
     # ---- sub-block 2: x_out = x_mid + dropout(ffn(ln2(x_mid)))
-    d = t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2])
+    d = dropped_in if dropped_in is not None else t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2])
     db2 = colsum_t(d)
     dw2 = matmul_t(d.t(), g1)                                           # [D,F]
     dg1 = matmul_t(d, w2)                                               # [N,F]
@@ -428,9 +463,9 @@ def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_
     db1 = colsum_t(df1)
     dw1 = matmul_t(df1.t(), h2)                                         # [F,D]
     dh2 = matmul_t(df1, w1)                                             # [N,D]
-    dx_mid, (dln2g, dln2b) = layernorm_bkwd2_t(dh2, (ln2g, ln2b), x_mid, residual=dloss_dx)
-    # ---- sub-block 1: x_mid = x_in + dropout(attn(ln1(x_in)))
-    d = t_dropout_bkwd2_t(dx_mid, None, train, p_gen_aux[1])
+    dx_mid, (dln2g, dln2b), d = layernorm_bkwd2_t(dh2, (ln2g, ln2b), x_mid, residual=dloss_dx,
+                                                  drop=(train, p_gen_aux[1], keep1))
+    # ---- sub-block 1: x_mid = x_in + dropout(attn(ln1(x_in))); d = dropout_bkwd(dx_mid) came with dx_mid
     dwo = matmul_t(d.t(), o2)                                           # [D,D]
     do2 = matmul_t(d, wo)                                               # [N,D] = [B,T,H,dh]
     v5 = qkv.view(B, T, H, 3, dh)
@@ -443,8 +478,15 @@ def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_
     attn_bwd_t(do4, q, k, v, o4, ms, ls, mask, train, p_gen_aux[0], out=outs)
     dwqkv = matmul_t(dqkv.t(), h1).view(H, 3, dh, D)                    # [H*3*dh, D]
     dh1 = matmul_t(dqkv, wqkv.view(H * 3 * dh, D))                      # [N,D]
-    dx_in, (dln1g, dln1b) = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid)
-    return dx_in, [dln1g, dln1b, dwqkv, dwo, dln2g, dln2b, dw1, db1, dw2, db2]
+    grads = None
+    if drop_out is not None:
+        dx_in, (dln1g, dln1b), dropped = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid, drop=drop_out)
+    else:
+        dx_in, (dln1g, dln1b) = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid)
+    grads = [dln1g, dln1b, dwqkv, dwo, dln2g, dln2b, dw1, db1, dw2, db2]
+    if drop_out is not None:
+        return dx_in, grads, dropped
+    return dx_in, grads
 
 
 def t_gpt2_tlayers_fwd3_t(params, y, mask, indices, train=True, p_gen_aux=None):
@@ -497,12 +539,23 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
     dbemb = colsum_t(dlog)
     dwemb = matmul_t(dlog.t(), h2d)                                     # [V,D]  LM-head weight grad
     dh = matmul_t(dlog, wemb)                                           # [N,D]
-    dx, (dlnfg, dlnfb) = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D))
+    # Every dropout backward acts on a gradient that a LayerNorm backward has just produced,
+    # so each LayerNorm backward also writes the dropped copy its consumer needs: the final
+    # norm for the last block's FFN dropout (seed 3L), block i's first norm for block i-1's
+    # FFN dropout (seed 3i) or, for block 0, for the embedding dropout (seed 0).
+    if L > 0:
+        dx, (dlnfg, dlnfb), dropped = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D),
+                                                       drop=(train, p_gen_aux[3 * L], layer_acts[L - 1][-1]))
+    else:
+        dx, (dlnfg, dlnfb), dropped = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D),
+                                                       drop=(train, p_gen_aux[0]))
     layer_grads = [None] * L
     for i in reversed(range(L)):
-        dx, layer_grads[i] = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train,
-                                                   p_gen_aux[1 + 3 * i:4 + 3 * i])
-    d = t_dropout_bkwd2_t(dx, None, train, p_gen_aux[0])                # [N,D]
+        dx, layer_grads[i], dropped = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train,
+                                                            p_gen_aux[1 + 3 * i:4 + 3 * i], dropped_in=dropped,
+                                                            drop_out=(train, p_gen_aux[3 * i],
+                                                                      layer_acts[i - 1][-1] if i > 0 else None))
+    d = dropped                                                         # [N,D] = dropout_bkwd(dx, seed 0)
     # positional table: sum over the batch (model_triton.py:2518 with indices = arange(T))
     dpos = torch.zeros_like(params[1][0])
     dpos[:T] = colsum_t(d.view(B, T * D)).view(T, D)

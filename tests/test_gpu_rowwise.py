@@ -133,3 +133,28 @@ def test_ce_all_labels_zero_is_nan(lo):
     x = torch.randn(4, 50, device=DEV)
     loss, cnt, dx = lo.t_avg_cross_entropy_loss_bkwd3_t(torch.zeros(4, dtype=torch.int64, device=DEV), x)
     assert torch.isnan(loss).all() and cnt.item() == 0 and (dx == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4096, 768), (33, 200), (7, 2048), (3, 5000)])
+def test_layernorm_bwd_with_dropout_output_matches_separate_calls(mt, dtype, shape):
+    """The LayerNorm backward that also emits dropout_bkwd(dx): bit-exact against the
+    LayerNorm backward followed by the dropout kernel, train and eval."""
+    g = gen(21)
+    dy, x, res = (randn(g, *shape, dtype=dtype).to(DEV) for _ in range(3))
+    gamma, beta = randn(g, shape[1], dtype=dtype).to(DEV), randn(g, shape[1], dtype=dtype).to(DEV)
+    for train in (True, False):
+        dx0, (dg0, db0) = mt.layernorm_bkwd2_t(dy, (gamma, beta), x, residual=res)
+        want = mt.t_dropout_bkwd2_t(dx0, None, train, 4242)
+        dx1, (dg1, db1), got = mt.layernorm_bkwd2_t(dy, (gamma, beta), x, residual=res, drop=(train, 4242))
+        assert torch.equal(dx0, dx1) and torch.equal(dg0, dg1) and torch.equal(db0, db1)
+        assert torch.equal(got, want)
+        # same again with the keep mask recorded by the forward dropout instead of recomputed
+        out, keep = mt.dropout_add_t(x, res, train, 4242, want_keep=True)
+        assert torch.equal(out, mt.dropout_add_t(x, res, train, 4242))
+        if keep is not None:
+            assert train and dtype == torch.bfloat16 and shape[1] % 8 == 0
+            _, _, got2 = mt.layernorm_bkwd2_t(dy, (gamma, beta), x, residual=res, drop=(train, 4242, keep))
+            assert torch.equal(got2, want)
+        else:
+            assert not (train and dtype == torch.bfloat16 and shape[1] % 8 == 0)
