@@ -19,6 +19,10 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# Measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this benchmark (commands, per-kernel table
+# and the copy-kernel scale factors: profiles/hbm_traffic__gpt2_b16_t1024_bf16_step.md): 228.3e6 read +
+# 69.3e6 written per GEMM launch, averaged over the forward, dX and dW products of a step.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 297.6e6
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
@@ -218,7 +222,9 @@ def main():
                    "global_batch": B, "seq_len": T, "step_tflop": round(total_flops / 1e12, 3),
                    "step_tflops_achieved": round(total_flops / 1e12 * value, 1)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic_note": "HBM bytes per GEMM launch (average over the 147 launches of a step) from rocprofv3 "
+                                     "FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy; algorithmic minimum 145.2e6",
                      "kernel": "gemm_kernel<bf16> (all %d launches of a step: fwd, dX, dW)" % (n_launch // args.steps),
                      "avg_launch_ms": round(gemm_ms / n_launch, 4),
                      "gflop_per_launch": round(gemm_flops / n_launch / 1e9, 2),
