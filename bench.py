@@ -201,7 +201,7 @@ def main():
     if not args.no_cpu:
         from oracle import gpt2 as ogpt2
         nthreads = torch.get_num_threads()
-        cb = 1
+        cb = 8                                   # about 15 s of CPU work on 16 host cores
         cparams = [[p.detach().to("cpu") for p in grp] for grp in master]
         cy = tokens[0, :cb].to("cpu")
         cmask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(cb, T, T)
