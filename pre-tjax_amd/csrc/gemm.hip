@@ -139,8 +139,10 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM
 // 3 first (the staging registers are free by then), so the single barrier of a step
 // finds no LDS read outstanding, and chunk 3 starts by reading chunk 0 of the other
 // buffer under its own MFMAs.  Loads past the last panel re-fetch it (discarded), so the
-// body has no branches and the staging registers stay plain values.
-template <typename T, int AMODE, int BMODE>
+// body has no branches and the staging registers stay plain values.  CLAMP: the tile
+// crosses the border of C; rows / columns past it re-read the last valid one (their
+// results are discarded by the bounds-checked epilogue).
+template <typename T, int AMODE, int BMODE, bool CLAMP>
 __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[TN][TM], char* __restrict__ smem,
                                               int row0, int col0, int kbeg, int nk) {
     constexpr int BK = BKB / (int)sizeof(T);
@@ -178,12 +180,12 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
 #define MV_A(I, LWA, LFA, P, KTF)                                                                         \
     do {                                                                                                  \
         LWA.template store_slice<I, 4>(sA + ((P) ^ 1) * A_BYTES, tid);                                    \
-        LFA.template load_fast_slice<I, 4>(A, g.a_row, g.a_k, row0, K0_OF(KTF), tid);                     \
+        LFA.template load_fast_slice<I, 4, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(KTF), tid, g.n);                     \
     } while (0)
 #define MV_B(I, LWB, LFB, P, KTF)                                                                         \
     do {                                                                                                  \
         LWB.template store_slice<I, 3>(sB + ((P) ^ 1) * B_BYTES, tid);                                    \
-        LFB.template load_fast_slice<I, 3>(B, g.b_row, g.b_k, col0, K0_OF(KTF), tid);                     \
+        LFB.template load_fast_slice<I, 3, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(KTF), tid, g.m);                     \
     } while (0)
 #define RF_STEP(P, LWA, LWB, LFA, LFB, KTF)                                                               \
     do {                                                                                                  \
@@ -211,10 +213,10 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
         MM(0, fx[0], 1); MM(1, fx[1], 1); MM(2, fx[2], 1); SB();                                          \
     } while (0)
 
-    la0.load_fast(A, g.a_row, g.a_k, row0, K0_OF(0), tid);
-    lb0.load_fast(B, g.b_row, g.b_k, col0, K0_OF(0), tid);
-    la1.load_fast(A, g.a_row, g.a_k, row0, K0_OF(1), tid);
-    lb1.load_fast(B, g.b_row, g.b_k, col0, K0_OF(1), tid);
+    la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(0), tid, g.n);
+    lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(0), tid, g.m);
+    la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(1), tid, g.n);
+    lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(1), tid, g.m);
     la0.store(sA, tid);
     lb0.store(sB, tid);
     __syncthreads();
@@ -390,14 +392,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
         const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
         const int nk_full = (kend - kbeg) / BK;  // whole panels
         if constexpr (VECTOR_OK) {
-            if (interior) {
-                gemm_run_fast<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, nk_full);
-                if (nk_full < nk) {
-                    __syncthreads();   // the pipelined loop leaves LDS reads in flight
-                    gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, nk_full, nk);
-                }
-            } else {
-                gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
+            // tiles that cross the border of C run the same pipeline with clamped row indices
+            if (interior) gemm_run_fast<T, AMODE, BMODE, false>(g, acc, smem, row0, col0, kbeg, nk_full);
+            else gemm_run_fast<T, AMODE, BMODE, true>(g, acc, smem, row0, col0, kbeg, nk_full);
+            if (nk_full < nk) {
+                __syncthreads();   // the pipelined loop leaves LDS reads in flight
+                gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, nk_full, nk);
             }
         } else {
             gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);

@@ -82,34 +82,55 @@ struct TileLoader {
     // offset that does not change along K.
     __device__ __forceinline__ void load_fast(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0, int k0,
                                               int tid) {
-        load_fast_slice<0, 1>(p, s_row, s_k, row0, k0, tid);
+        load_fast_slice<0, 1, false>(p, s_row, s_k, row0, k0, tid, 0);
     }
 
     // Slice I of N of load_fast (every N-th load), so that a caller can spread the loads of
-    // one panel between other work.
-    template <int I, int N>
+    // one panel between other work.  CLAMP: the panel may extend past the last row of the
+    // operand (nrows); rows past it re-read the last valid row / row vector instead, so the
+    // loads stay straight-line and in bounds and the caller discards those rows' results.
+    template <int I, int N, bool CLAMP>
     __device__ __forceinline__ void load_fast_slice(const T* __restrict__ p, int64_t s_row, int64_t s_k, int row0,
-                                                    int k0, int tid) {
+                                                    int k0, int tid, int nrows) {
         static_assert(MODE != GENERIC, "GENERIC panels have no vector path");
         // Byte addressing: wave-uniform 64-bit base + one unsigned 32-bit lane offset.
         if constexpr (MODE == KMAJOR) {
-            const char* ub = reinterpret_cast<const char*>(p + (int64_t)row0 * s_row + k0);   // uniform
-            const uint32_t loff = ((uint32_t)(tid >> 3) * (uint32_t)s_row + (tid & 7) * VEC) * (uint32_t)sizeof(T);
+            if constexpr (!CLAMP) {
+                const char* ub = reinterpret_cast<const char*>(p + (int64_t)row0 * s_row + k0);   // uniform
+                const uint32_t loff = ((uint32_t)(tid >> 3) * (uint32_t)s_row + (tid & 7) * VEC) * (uint32_t)sizeof(T);
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                if (i % N != I) continue;
-                if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS))
-                    r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row * (int64_t)sizeof(T) + loff);
+                for (int i = 0; i < NV; ++i) {
+                    if (i % N != I) continue;
+                    if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS))
+                        r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row * (int64_t)sizeof(T) + loff);
+                }
+            } else {
+                const char* ub = reinterpret_cast<const char*>(p + k0);                            // uniform
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    if (i % N != I) continue;
+                    if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS)) {
+                        int row = row0 + (tid >> 3) + RP * i;
+                        row = row < nrows ? row : nrows - 1;
+                        r[i] = *reinterpret_cast<const u32x4*>(
+                            ub + ((int64_t)row * s_row + (tid & 7) * VEC) * (int64_t)sizeof(T));
+                    }
+                }
             }
         } else {
             const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
-            const char* ub = reinterpret_cast<const char*>(p + (int64_t)k0 * s_k + row0);     // uniform
+            const char* ub = reinterpret_cast<const char*>(p + (int64_t)k0 * s_k + (CLAMP ? 0 : row0));   // uniform
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
                 if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
-                    const uint32_t loff = ((uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k +
-                                           ((b % JB) * 8 + jc_lo) * VEC) * (uint32_t)sizeof(T);
+                    int rowv = ((b % JB) * 8 + jc_lo) * VEC;               // first row of the lane's row vector
+                    if constexpr (CLAMP) {
+                        const int lastv = ((nrows - 1) / VEC) * VEC;        // a .t() view's pitch covers this vector
+                        rowv = row0 + rowv < lastv ? row0 + rowv : lastv;
+                    }
+                    const uint32_t loff =
+                        ((uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k + (uint32_t)rowv) * (uint32_t)sizeof(T);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         if ((qi * 4 + i) % N != I) continue;
