@@ -7,7 +7,9 @@
 // the big products fill the 256 CUs in whole rounds.  K advances in panels of 128 BYTES
 // per row (64 bf16 / 32 fp32), double-buffered in LDS (2 x 56 KiB): while the MFMAs
 // consume buffer p, the next panels travel HBM -> registers -> buffer p^1, one barrier
-// per step; two wavefronts per SIMD overlap one's MFMAs with the other's copies.
+// per step; two wavefronts per SIMD overlap one's MFMAs with the other's copies.  The
+// kernel is persistent (one workgroup per CU); without a K split the panel pipeline runs
+// on across a workgroup's tiles, so only its first tile pays the load latency up front.
 //
 // LDS panels and their swizzle are described in mma_tile.h.  Operands whose contiguous
 // axis is K are copied 16 bytes at a time; operands whose contiguous axis is the
@@ -60,6 +62,7 @@ struct GemmArgs {
     int64_t c_rs;
     int k_per_split;      // multiple of BK
     int splits;
+    int stream;           // no K split and K is a whole even number of panels: tiles are pipelined back to back
     int vec_out;          // every output (C, pre-activation, partials) and the bias allow aligned 16-byte rows
     int epilogue;
 };
@@ -165,6 +168,8 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
 
 #define SB() __builtin_amdgcn_sched_barrier(0)
 #define K0_OF(KT) (kbeg + ((KT) < last ? (KT) : last) * BK)
+#define ROW_A(KT) row0
+#define ROW_B(KT) col0
 #define RD_A(P, C, BUF)                                                                                   \
     do {                                                                                                  \
         _Pragma("unroll") for (int t = 0; t < TM; ++t)                                                    \
@@ -180,12 +185,12 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
 #define MV_A(I, LWA, LFA, P, KTF)                                                                         \
     do {                                                                                                  \
         LWA.template store_slice<I, 4>(sA + ((P) ^ 1) * A_BYTES, tid);                                    \
-        LFA.template load_fast_slice<I, 4, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(KTF), tid, g.n);                     \
+        LFA.template load_fast_slice<I, 4, CLAMP>(A, g.a_row, g.a_k, ROW_A(KTF), K0_OF(KTF), tid, g.n);   \
     } while (0)
 #define MV_B(I, LWB, LFB, P, KTF)                                                                         \
     do {                                                                                                  \
         LWB.template store_slice<I, 3>(sB + ((P) ^ 1) * B_BYTES, tid);                                    \
-        LFB.template load_fast_slice<I, 3, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(KTF), tid, g.m);                     \
+        LFB.template load_fast_slice<I, 3, CLAMP>(B, g.b_row, g.b_k, ROW_B(KTF), K0_OF(KTF), tid, g.m);   \
     } while (0)
 #define RF_STEP(P, LWA, LWB, LFA, LFB, KTF)                                                               \
     do {                                                                                                  \
@@ -227,14 +232,9 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
         RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
     }
     if (kt < nk) RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
-#undef SB
 #undef K0_OF
-#undef RD_A
-#undef RD_B
-#undef MM
-#undef RF_STEP
-#undef MV_A
-#undef MV_B
+#undef ROW_A
+#undef ROW_B
 }
 
 // LDS: two operand panel buffers (2 x 56 KiB) followed by one 6 KiB output staging area per
@@ -246,20 +246,28 @@ constexpr int SMEM_BYTES = PANEL_BYTES + (GEMM_THREADS / 64) * STAGE_BYTES;
 
 // Writes the wave's 64x96 accumulator block to `dst` (row pitch dst_rs elements of OUT)
 // through the wave-private staging area: 32 rows per pass for 2-byte outputs, 16 for
-// 4-byte outputs.  A staged row is 96 outputs; its 16-byte chunks are rotated by the row
-// number (in place of padding) so that the 32 rows of a write land in different banks.
+// 4-byte outputs.  A staged row is 96 outputs = three groups of 32 columns (LPR 16-byte
+// chunks each); inside a group the chunk index is XORed with bits of the row number, which
+// spreads both the column-wise writes of the accumulator layout and the row-wise reads
+// over all banks and keeps every address a per-lane base plus a compile-time offset.
+// The write-back gives each row of a group to LPR consecutive lanes (64 or 128 contiguous
+// bytes per row, 16 or 8 rows per store instruction).
+// BIAS: add g.bias here (false when the accumulators were started from the bias).
+// ACT: apply the GELU when the epilogue asks for it.
 // FULL: the tile lies inside C and dst / bias are vector-aligned, so the write-back is
 // straight-line 16-byte stores; otherwise every element is bounds-checked.  The two
 // variants are separate instantiations on purpose: when both appear behind one per-lane
 // condition the compiler merges them into partial (12 + 2 + 2 byte) stores.  The global
 // stores are not waited for.
-template <typename OUT, typename T, bool EPILOGUE, bool NO_ACT, bool FULL>
+template <typename OUT, typename T, bool BIAS, bool ACT, bool FULL>
 __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
                                                  int row0, int col0, OUT* __restrict__ dst, int64_t dst_rs) {
     constexpr int RB = 96 * (int)sizeof(OUT);                    // bytes per staged row
-    constexpr int NC = RB / 16;                                  // 16-byte chunks per row
     constexpr int ROWS = STAGE_BYTES / RB;                       // rows per pass
     constexpr int V = 16 / (int)sizeof(OUT);                     // elements per 16-byte vector
+    constexpr int LPR = 32 / V;                                  // chunks per 32-column group = lanes per row
+    constexpr int KS = sizeof(OUT) == 2 ? 2 : 1;                 // swizzle key = (row >> KS) & (LPR - 1)
+    constexpr int RPI = 64 / LPR;                                // rows per store instruction
     static_assert(ROWS == 32 || ROWS == 16, "staging pass");
     const int tid = fresh_tid();
     const int lane = tid & 63, wave = tid >> 6;
@@ -269,13 +277,12 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
     const int gcol0 = col0 + wn * 96;
     const int grow0 = row0 + wm * 64;
     const int sr = lr & (ROWS - 1);                              // staged row of this lane
-    const int srot = sr % NC;
-    const bool has_bias = EPILOGUE && g.epilogue != PTJ_EPI_NONE;
-    const bool act = EPILOGUE && !NO_ACT && g.epilogue == PTJ_EPI_BIAS_GELU;
+    const bool has_bias = BIAS && g.epilogue != PTJ_EPI_NONE;
+    const bool act = ACT && g.epilogue == PTJ_EPI_BIAS_GELU;
 
     // bias of this lane's 12 column quads
     float bias[TN * 4][4];
-    if constexpr (EPILOGUE) {
+    if constexpr (BIAS) {
 #pragma unroll
         for (int q = 0; q < TN * 4; ++q) {
             const int cc = (q >> 2) * 32 + (q & 3) * 8 + lg * 4;
@@ -292,6 +299,21 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
             }
         }
     }
+    // write side: the lane's 4 columns of quad i4 sit in chunk (i4 [*2 + lg]) of group tn
+    const int wkey = (sr >> KS) & (LPR - 1);
+    char* wrow = stage + sr * RB + (sizeof(OUT) == 2 ? lg * 8 : 0);
+    int woff[4];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) woff[i4] = (((sizeof(OUT) == 2 ? i4 : i4 * 2 + lg) ^ wkey) << 4);
+    // read side: lane -> row (lane / LPR) of the instruction's RPI rows, chunk lane % LPR
+    const int rrow = lane / LPR, rch = lane % LPR;
+    const char* rbase[ROWS / RPI];
+#pragma unroll
+    for (int h = 0; h < ROWS / RPI; ++h) {
+        const int r = h * RPI + rrow;
+        rbase[h] = stage + r * RB + ((rch ^ ((r >> KS) & (LPR - 1))) << 4);
+    }
+    OUT* gbase = dst + (int64_t)(grow0 + rrow) * dst_rs + gcol0 + rch * V;
 #pragma unroll
     for (int pass = 0; pass < 64 / ROWS; ++pass) {
         const int tm = pass * ROWS / 32;
@@ -300,48 +322,207 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
-                const int cc = tn * 32 + i4 * 8 + lg * 4;        // first of 4 columns, block-relative
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = acc[tn][tm][i4 * 4 + e];
-                if constexpr (EPILOGUE) {
+                if constexpr (BIAS) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) o[e] += bias[tn * 4 + i4][e];
+                }
+                if constexpr (ACT) {
                     if (act) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) o[e] = gelu_f(o[e]);
                     }
                 }
-                const int byte = cc * (int)sizeof(OUT);
-                int ch = (byte >> 4) + srot;
-                ch = ch >= NC ? ch - NC : ch;
-                if (ROWS == 32 || mine)
-                    store_vec<OUT, 4>(reinterpret_cast<OUT*>(stage + sr * RB + (ch << 4) + (byte & 15)), o);
+                if (ROWS == 32 || mine) store_vec<OUT, 4>(reinterpret_cast<OUT*>(wrow + tn * (LPR * 16) + woff[i4]), o);
             }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   // the wave re-reads only its own area
 #pragma unroll
-        for (int it = 0; it < ROWS * NC / 64; ++it) {
-            const int v = it * 64 + lane;
-            const int r = v / NC, c = v % NC;
-            int ch = c + r % NC;
-            ch = ch >= NC ? ch - NC : ch;
-            const int grow = grow0 + pass * ROWS + r;
-            const int gcol = gcol0 + c * V;
-            const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(stage + r * RB + (ch << 4));
-            OUT* p = dst + (int64_t)grow * dst_rs + gcol;
-            if constexpr (FULL) {
-                *reinterpret_cast<Pack<OUT, V>*>(p) = val;
-            } else {
-                if (grow < g.n) {
+        for (int h = 0; h < ROWS / RPI; ++h)
 #pragma unroll
-                    for (int e = 0; e < V; ++e)
-                        if (gcol + e < g.m) p[e] = val.v[e];
+            for (int g3 = 0; g3 < 3; ++g3) {
+                const int r = pass * ROWS + h * RPI;             // block row of the instruction's first row
+                const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(rbase[h] + g3 * (LPR * 16));
+                OUT* p = gbase + (int64_t)r * dst_rs + g3 * 32;
+                if constexpr (FULL) {
+                    *reinterpret_cast<Pack<OUT, V>*>(p) = val;
+                } else {
+                    if (grow0 + r + rrow < g.n) {
+                        const int gcol = gcol0 + g3 * 32 + rch * V;
+#pragma unroll
+                        for (int e = 0; e < V; ++e)
+                            if (gcol + e < g.m) p[e] = val.v[e];
+                    }
                 }
             }
-        }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     }
 }
+
+// Work item -> origin of its C tile: ids are regrouped so that the items of one XCD (id mod
+// 8) cover a contiguous range of tiles, then walked in groups of 8 tile-rows.
+#ifndef PTJ_GEMM_GROUP
+#define PTJ_GEMM_GROUP 8
+#endif
+__device__ __forceinline__ void tile_origin(int pid, int total, int num_m, int num_n, int& row0, int& col0) {
+    {
+        const int chunk = total >> 3, rem = total & 7, x = pid & 7;
+        pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
+    }
+    constexpr int GROUP = PTJ_GEMM_GROUP;
+    const int width = GROUP * num_n;
+    const int group_id = pid / width;
+    const int first_m = group_id * GROUP;
+    const int gsz = (num_m - first_m) < GROUP ? (num_m - first_m) : GROUP;
+    const int tile_m = first_m + (pid % width) % gsz;
+    const int tile_n = (pid % width) / gsz;
+    row0 = tile_m * BM;
+    col0 = tile_n * BN;
+}
+
+// Epilogue of one tile.  acc[tn][tm][i] of lane (lr, lg) is
+//   C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)].
+// Bias / GELU are applied in registers, the block is converted to the output type,
+// staged in the wave-private LDS area and written back as 16-byte vectors that run
+// along whole 96-column rows.  Only wave-local ordering is needed.
+template <typename T, bool BIAS>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
+                                              int row0, int col0, int z) {
+    const bool full = row0 + BM <= g.n && col0 + BN <= g.m && g.vec_out;
+    if (g.partial != nullptr) {
+        float* part = g.partial + (int64_t)z * g.n * (int64_t)g.m;
+        if (full) gemm_store_block<float, T, false, false, true>(g, acc, smem, row0, col0, part, g.m);
+        else gemm_store_block<float, T, false, false, false>(g, acc, smem, row0, col0, part, g.m);
+    } else if (full) {
+        if (g.c_aux != nullptr)
+            gemm_store_block<T, T, BIAS, false, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+        gemm_store_block<T, T, BIAS, true, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+    } else {
+        if (g.c_aux != nullptr)
+            gemm_store_block<T, T, BIAS, false, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+        gemm_store_block<T, T, BIAS, true, false>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+    }
+}
+
+// Bias of this lane's 12 column quads of the tile at column col0, in storage type (zeros
+// without a bias).  CLAMP: the tile may cross the right border; columns past it re-read
+// the last valid one.
+template <typename T, bool CLAMP>
+__device__ __forceinline__ void load_bias_quads(const GemmArgs& g, int col0, Pack<T, 4> (&b)[TN * 4]) {
+    const int tid = fresh_tid();
+    const int lg = (tid & 63) >> 5, wn = (tid >> 6) % WAVES_N;
+    const int gcol0 = col0 + wn * 96 + lg * 4;
+    const T* bias = (const T*)g.bias;
+    if (g.epilogue == PTJ_EPI_NONE) {
+#pragma unroll
+        for (int q = 0; q < TN * 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[q].v[e] = from_f32<T>(0.f);
+        return;
+    }
+    bool whole = true;
+    if constexpr (CLAMP) whole = col0 + BN <= g.m;
+    if (whole) {
+#pragma unroll
+        for (int q = 0; q < TN * 4; ++q)
+            b[q] = *reinterpret_cast<const Pack<T, 4>*>(bias + gcol0 + (q >> 2) * 32 + (q & 3) * 8);
+    } else {
+#pragma unroll
+        for (int q = 0; q < TN * 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int c = gcol0 + (q >> 2) * 32 + (q & 3) * 8 + e;
+                b[q].v[e] = bias[c < g.m ? c : g.m - 1];
+            }
+    }
+}
+
+// The pipelined loop of gemm_run_fast carried across the tiles of a workgroup (no K
+// split, K a whole even number of panels): the two panel fetches that run past the end
+// of a tile bring in the first two panels of the workgroup's next tile instead of
+// re-reading the last one, so after the last step the LDS buffer, the staging registers
+// and the operand registers are exactly in the state the loop expects on entry.  The
+// epilogue (which stages through its own LDS area) runs between two tiles while those
+// loads are in flight.  A workgroup without a next tile re-fetches its own first panels.
+// The accumulators start from the bias (loaded while the previous tile's epilogue runs)
+// instead of zero, so the epilogue neither waits for bias loads nor adds them.
+template <typename T, int AMODE, int BMODE, bool CLAMP>
+__device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict__ smem) {
+    constexpr int BK = BKB / (int)sizeof(T);
+    constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+    const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
+    const int total = num_m * num_n;
+    const int nk = g.k / BK;
+    const T* A = (const T*)g.a;
+    const T* B = (const T*)g.b;
+    char* sA = smem;
+    char* sB = smem + 2 * A_BYTES;
+    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1;
+    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1;
+    typename Frag<T>::type fa[2][TM], fb[TN], fx[TN];
+    int item = blockIdx.x;
+    int row0, col0;
+    tile_origin(item, total, num_m, num_n, row0, col0);
+    Pack<T, 4> braw[TN * 4];
+    load_bias_quads<T, CLAMP>(g, col0, braw);
+    {
+        const int tid = fresh_tid();
+        const int lane = tid & 63, wave = tid >> 6;
+        const int lr = lane & 31, lg = lane >> 5;
+        const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
+        la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, 0, tid, g.n);
+        lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, 0, tid, g.m);
+        la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, BK, tid, g.n);
+        lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, BK, tid, g.m);
+        la0.store(sA, tid);
+        lb0.store(sB, tid);
+        __syncthreads();
+        RD_A(0, 0, 0); RD_B(fb[0], 0, 0, 0); RD_B(fb[1], 0, 0, 1); RD_B(fb[2], 0, 0, 2); SB();
+    }
+    for (;;) {
+        const int nitem = item + (int)gridDim.x;
+        const bool more = nitem < total;
+        int nrow0, ncol0;
+        tile_origin(more ? nitem : item, total, num_m, num_n, nrow0, ncol0);
+        f32x16 acc[TN][TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = to_f32(braw[i * 4 + (e >> 2)].v[e & 3]);
+        {
+            const int tid = fresh_tid();
+            const int lane = tid & 63, wave = tid >> 6;
+            const int lr = lane & 31, lg = lane >> 5;
+            const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
+#define K0_OF(KT) (((KT) < nk ? (KT) : (KT) - nk) * BK)
+#define ROW_A(KT) ((KT) < nk ? row0 : nrow0)
+#define ROW_B(KT) ((KT) < nk ? col0 : ncol0)
+            for (int kt = 0; kt < nk; kt += 2) {
+                RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+                RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+            }
+#undef K0_OF
+#undef ROW_A
+#undef ROW_B
+        }
+        load_bias_quads<T, CLAMP>(g, ncol0, braw);
+        gemm_epilogue<T, false>(g, acc, smem, row0, col0, 0);
+        if (!more) break;
+        item = nitem;
+        row0 = nrow0;
+        col0 = ncol0;
+    }
+}
+#undef SB
+#undef RD_A
+#undef RD_B
+#undef MM
+#undef RF_STEP
+#undef MV_A
+#undef MV_B
 
 // Persistent kernel: workgroup b handles work items b, b + gridDim.x, ... where an item is
 // one (C tile, K split) pair; the stores of a finished tile drain while the next tile's
@@ -350,31 +531,22 @@ template <typename T, int AMODE, int BMODE>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
-    
+    constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
+    if constexpr (VECTOR_OK) {
+        if (g.stream) {
+            if (g.n % BM == 0 && g.m % BN == 0) gemm_stream<T, AMODE, BMODE, false>(g, smem);
+            else gemm_stream<T, AMODE, BMODE, true>(g, smem);
+            return;
+        }
+    }
 
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     const int total = num_m * num_n;
     const int work = total * g.splits;
     for (int item = blockIdx.x; item < work; item += gridDim.x) {
         const int z = item / total;
-        int pid = item - z * total;
-        // ---- work item -> tile: regroup so that the items of one XCD (id mod 8) cover a
-        // contiguous range of tiles, then walk groups of 8 tile-rows.
-        {
-            const int chunk = total >> 3, rem = total & 7, x = pid & 7;
-            pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
-        }
-#ifndef PTJ_GEMM_GROUP
-#define PTJ_GEMM_GROUP 8
-#endif
-        constexpr int GROUP = PTJ_GEMM_GROUP;
-        const int width = GROUP * num_n;
-        const int group_id = pid / width;
-        const int first_m = group_id * GROUP;
-        const int gsz = (num_m - first_m) < GROUP ? (num_m - first_m) : GROUP;
-        const int tile_m = first_m + (pid % width) % gsz;
-        const int tile_n = (pid % width) / gsz;
-        const int row0 = tile_m * BM, col0 = tile_n * BN;
+        int row0, col0;
+        tile_origin(item - z * total, total, num_m, num_n, row0, col0);
 
         const int kbeg = z * g.k_per_split;
         const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
@@ -388,7 +560,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
         const bool interior = row0 + BM <= g.n && col0 + BN <= g.m;
         const int nk_full = (kend - kbeg) / BK;  // whole panels
         if constexpr (VECTOR_OK) {
@@ -402,26 +573,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
         } else {
             gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
         }
-
-        // ---- epilogue.  acc[tn][tm][i] of lane (lr, lg) is
-        //   C[wm*64 + tm*32 + lr][wn*96 + tn*32 + (i/4)*8 + lg*4 + (i%4)].
-        // Bias / GELU are applied in registers, the block is converted to the output type,
-        // staged in the wave-private LDS area and written back as 16-byte vectors that run
-        // along whole 96-column rows.  Only wave-local ordering is needed.
-        const bool full = interior && g.vec_out;
-        if (g.partial != nullptr) {
-            float* part = g.partial + (int64_t)z * g.n * (int64_t)g.m;
-            if (full) gemm_store_block<float, T, false, false, true>(g, acc, smem, row0, col0, part, g.m);
-            else gemm_store_block<float, T, false, false, false>(g, acc, smem, row0, col0, part, g.m);
-        } else if (full) {
-            if (g.c_aux != nullptr)
-                gemm_store_block<T, T, true, true, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
-            gemm_store_block<T, T, true, false, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
-        } else {
-            if (g.c_aux != nullptr)
-                gemm_store_block<T, T, true, true, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
-            gemm_store_block<T, T, true, false, false>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
-        }
+        gemm_epilogue<T, true>(g, acc, smem, row0, col0, z);
     }
 }
 
@@ -561,6 +713,8 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
         g.vec_out = ok ? 1 : 0;
     }
     g.partial = splits > 1 ? (float*)workspace : nullptr;
+    // streamed tiles need whole, evenly many K panels (the two-step loop body) and vector-aligned outputs
+    g.stream = (splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
 }

@@ -105,15 +105,21 @@ struct TileLoader {
                         r[i] = *reinterpret_cast<const u32x4*>(ub + (int64_t)(RP * i) * s_row * (int64_t)sizeof(T) + loff);
                 }
             } else {
-                const char* ub = reinterpret_cast<const char*>(p + k0);                            // uniform
+                // rows past the operand's last one re-read it; both addresses are a uniform
+                // base plus a 32-bit lane offset, so the clamp costs a compare and selects
+                const int64_t rstep = s_row * (int64_t)sizeof(T);
+                const char* ub = reinterpret_cast<const char*>(p + (int64_t)row0 * s_row + k0);   // uniform
+                const int lim = nrows - 1 - row0;
+                const char* last = ub + (int64_t)lim * rstep;                                      // uniform
+                const uint32_t col = (uint32_t)((tid & 7) * VEC * (int)sizeof(T));
+                const uint32_t loff = (uint32_t)(tid >> 3) * (uint32_t)s_row * (uint32_t)sizeof(T) + col;
 #pragma unroll
                 for (int i = 0; i < NV; ++i) {
                     if (i % N != I) continue;
                     if ((ROWS % RP == 0) || ((tid >> 3) + RP * i < ROWS)) {
-                        int row = row0 + (tid >> 3) + RP * i;
-                        row = row < nrows ? row : nrows - 1;
-                        r[i] = *reinterpret_cast<const u32x4*>(
-                            ub + ((int64_t)row * s_row + (tid & 7) * VEC) * (int64_t)sizeof(T));
+                        const bool in = (tid >> 3) + RP * i <= lim;
+                        const char* a = in ? ub + (int64_t)(RP * i) * rstep + loff : last + col;
+                        r[i] = *reinterpret_cast<const u32x4*>(a);
                     }
                 }
             }
