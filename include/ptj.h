@@ -70,10 +70,13 @@ int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const vo
  * (model_triton.py:2021-2024, 2175-2178) without another pass over dx.  Bit-identical to
  * ptj_layernorm_bwd followed by ptj_dropout.  `keep_bytes` (nullable) are the keep bits
  * that ptj_dropout_add_keep recorded for the same (seed, shape); with them the mask is
- * read instead of recomputed (2-byte element types only). */
+ * read instead of recomputed (2-byte element types only).  `dropped_colsum` (nullable,
+ * [cols]; needs dropped and dgamma) receives the column sums of the stored `dropped`: the
+ * `.sum(dim=0)` bias gradient of the linear layer that `dropped` is the output gradient of
+ * (model_triton.py:426), from the same two-stage reduction as dgamma/dbeta. */
 int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, const void* residual,
                               void* dx, void* dgamma, void* dbeta,
-                              void* dropped, int drop_train, int64_t drop_seed,
+                              void* dropped, void* dropped_colsum, int drop_train, int64_t drop_seed,
                               const void* keep_bytes,
                               void* workspace, size_t workspace_bytes,
                               int64_t rows, int64_t cols, int64_t dy_row_stride, int64_t x_row_stride,
@@ -90,6 +93,13 @@ int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes
  * Replace t_gelu_fwd_k/_t (model_triton.py:237-260) and t_gelu_bkwd2_k/_t (:274-304). */
 int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
 int ptj_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype, void* stream);
+/* GELU backward on [rows, cols] (contiguous) that also returns the column sums of dx:
+ * dx = dy * gelu'(x), colsum[c] = sum_r dx[r, c] over the stored (rounded) values -- the
+ * gradient of the bias in front of the GELU (t_gelu_bkwd2_t followed by the `.sum(dim=0)`
+ * of t_linear_bkwd2_p, model_triton.py:296-304 and :426) in one pass over dx.
+ * `workspace`: ptj_colsum_workspace_bytes(rows, cols) bytes. */
+int ptj_gelu_bwd_colsum(const void* dy, const void* x, void* dx, void* colsum, void* workspace,
+                        size_t workspace_bytes, int64_t rows, int64_t cols, int dtype, void* stream);
 
 /* Dropout, rate 0.1, non-inverted: train != 0 -> y = keep ? x : 0 with
  * keep = tl.rand(seed + row, col) > 0.1 (Philox4x32-10); train == 0 -> y = 0.9*x.

@@ -24,12 +24,13 @@ SIGNATURES = {
     "ptj_layernorm_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_layernorm_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64, _int, _p]),
-    "ptj_layernorm_bwd_dropout": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _int, _i64, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64,
+    "ptj_layernorm_bwd_dropout": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _i64, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64,
                                          _int, _p]),
     "ptj_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_colsum": (_int, [_p, _p, _p, _sz, _i64, _i64, _i64, _int, _p]),
     "ptj_gelu_fwd": (_int, [_p, _p, _i64, _int, _p]),
     "ptj_gelu_bwd": (_int, [_p, _p, _p, _i64, _int, _p]),
+    "ptj_gelu_bwd_colsum": (_int, [_p, _p, _p, _p, _p, _sz, _i64, _i64, _int, _p]),
     "ptj_dropout": (_int, [_p, _p, _i64, _i64, _i64, _i64, _int, _i64, _int, _p]),
     "ptj_dropout_add": (_int, [_p, _p, _p, _i64, _i64, _int, _i64, _int, _p]),
     "ptj_dropout_add_keep": (_int, [_p, _p, _p, _p, _i64, _i64, _int, _i64, _int, _p]),

@@ -103,7 +103,9 @@ template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
 __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
     T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs,
-    T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep) {
+    T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep, int np) {
+    // np: partial sums per workgroup and column: dgamma, dbeta and, with np == 3, the
+    // column sums of the `drop` output
     __shared__ float smem[16];
     constexpr int RPB = LnBwdGeom<TPR>::ROWS_PER_BLOCK;
     const int t = threadIdx.x % TPR;
@@ -111,12 +113,12 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const int nvec = cols / VEC;
     RowRegs<T, VEC, TPR, ITERS> g;
     if constexpr (DX) g.load(gamma, nvec, t, 0.f);
-    float acc_g[ITERS][VEC], acc_b[ITERS][VEC];
+    float acc_g[ITERS][VEC], acc_b[ITERS][VEC], acc_d[ITERS][VEC];
     if constexpr (DGB) {
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc_g[it][j] = acc_b[it][j] = 0.f;
+            for (int j = 0; j < VEC; ++j) acc_g[it][j] = acc_b[it][j] = acc_d[it][j] = 0.f;
     }
     const float inv_n = 1.0f / (float)cols;
     const float inv_nm1 = 1.0f / (float)(cols - 1);
@@ -207,6 +209,9 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                     for (int j = 0; j < VEC; ++j) {
                         const float r = to_f32(from_f32<T>(d.v[it][j]));
                         d.v[it][j] = drop_train ? (((bits >> j) & 1u) ? r : 0.f) : r * 0.9f;
+                        if constexpr (DGB) {
+                            if (np == 3) acc_d[it][j] += to_f32(from_f32<T>(d.v[it][j]));   // the stored value
+                        }
                     }
                 }
                 d.store(drop + row * (int64_t)cols, nvec, t);
@@ -216,10 +221,11 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     if constexpr (DGB) {
         // One partial per workgroup.  With several row slots per workgroup the slots are
         // folded through LDS in slot order (deterministic).
-        float* pg = part + (int64_t)blockIdx.x * 2 * (int64_t)cols;
+        float* pg = part + (int64_t)blockIdx.x * np * (int64_t)cols;
         float* pb = pg + cols;
+        float* pd = pb + cols;
         if constexpr (RPB > 1) {
-            __shared__ float red[2][LN_BWD_MAX_WAVE_COLS];
+            __shared__ float red[3][LN_BWD_MAX_WAVE_COLS];
             for (int s = 0; s < RPB; ++s) {
                 if (sub == s) {
 #pragma unroll
@@ -231,6 +237,7 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                                 const int c = vi * VEC + j;
                                 red[0][c] = s == 0 ? acc_g[it][j] : red[0][c] + acc_g[it][j];
                                 red[1][c] = s == 0 ? acc_b[it][j] : red[1][c] + acc_b[it][j];
+                                red[2][c] = s == 0 ? acc_d[it][j] : red[2][c] + acc_d[it][j];
                             }
                         }
                     }
@@ -240,6 +247,7 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
             for (int c = threadIdx.x; c < cols; c += LnBwdGeom<TPR>::BLOCK) {
                 pg[c] = red[0][c];
                 pb[c] = red[1][c];
+                if (np == 3) pd[c] = red[2][c];
             }
         } else {
 #pragma unroll
@@ -250,6 +258,7 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                     for (int j = 0; j < VEC; ++j) {
                         pg[vi * VEC + j] = acc_g[it][j];
                         pb[vi * VEC + j] = acc_b[it][j];
+                        if (np == 3) pd[vi * VEC + j] = acc_d[it][j];
                     }
                 }
             }
@@ -285,16 +294,17 @@ __device__ __forceinline__ float reduce_partials(const float* __restrict__ col_b
     return r;
 }
 
-// Second stage: out[which][c] = sum_p part[p][which][c], fixed order.  grid = (ceil(cols/32), 2).
+// Second stage: out[which][c] = sum_p part[p][which][c], fixed order.  grid = (ceil(cols/32), np)
+// with np = 2 (dgamma, dbeta) or 3 (and the column sums of the dropped output).
 template <typename T>
 __global__ __launch_bounds__(RED_THREADS) void layernorm_bwd_reduce_kernel(const float* __restrict__ part, int nparts,
                                                                             int cols, T* __restrict__ dgamma,
-                                                                            T* __restrict__ dbeta) {
+                                                                            T* __restrict__ dbeta, T* __restrict__ dsum) {
     __shared__ float sm[32][33];
     const int c = blockIdx.x * 32 + (threadIdx.x & 31);
-    const int which = blockIdx.y;
-    const float r = reduce_partials(part + (int64_t)which * cols + c, 2 * (int64_t)cols, nparts, c < cols, sm);
-    if ((threadIdx.x >> 5) == 0 && c < cols) (which == 0 ? dgamma : dbeta)[c] = from_f32<T>(r);
+    const int which = blockIdx.y, np = gridDim.y;
+    const float r = reduce_partials(part + (int64_t)which * cols + c, np * (int64_t)cols, nparts, c < cols, sm);
+    if ((threadIdx.x >> 5) == 0 && c < cols) (which == 0 ? dgamma : which == 1 ? dbeta : dsum)[c] = from_f32<T>(r);
 }
 
 // ---------------------------------------------------------------------------------
@@ -487,6 +497,56 @@ __global__ __launch_bounds__(RED_THREADS) void colsum_stage2_kernel(const float*
     if ((threadIdx.x >> 5) == 0 && c < cols) out[c] = from_f32<T>(r);
 }
 
+// GELU backward with the column sums of its own output (the bias gradient of the linear
+// layer in front of the GELU) in the colsum_stage1 geometry: block (bx, by) handles rows
+// [by*rps, (by+1)*rps) of its 128*VEC columns, writes dx and leaves the sums of the stored
+// (storage-rounded) dx values in part[by][col].
+template <typename T, int VEC>
+__global__ __launch_bounds__(128) void gelu_bwd_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                              T* __restrict__ dx, float* __restrict__ part,
+                                                              int64_t rows, int cols, int rows_per_split) {
+    const int c0 = (blockIdx.x * 128 + threadIdx.x) * VEC;
+    if (c0 >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+    const int64_t r1 = r0 + rows_per_split < rows ? r0 + rows_per_split : rows;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    constexpr int U = 4;   // independent rows in flight per thread
+    int64_t r = r0;
+    for (; r + U <= r1; r += U) {
+        float v[U][VEC], d[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            load_vec<T, VEC>(x + (r + u) * (int64_t)cols + c0, v[u]);
+            load_vec<T, VEC>(dy + (r + u) * (int64_t)cols + c0, d[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                d[u][j] = to_f32(from_f32<T>(d[u][j] * gelu_grad_f(v[u][j])));
+                acc[j] += d[u][j];
+            }
+            store_vec<T, VEC>(dx + (r + u) * (int64_t)cols + c0, d[u]);
+        }
+    }
+    for (; r < r1; ++r) {
+        float v[VEC], d[VEC];
+        load_vec<T, VEC>(x + r * (int64_t)cols + c0, v);
+        load_vec<T, VEC>(dy + r * (int64_t)cols + c0, d);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            d[j] = to_f32(from_f32<T>(d[j] * gelu_grad_f(v[j])));
+            acc[j] += d[j];
+        }
+        store_vec<T, VEC>(dx + r * (int64_t)cols + c0, d);
+    }
+    float* dst = part + (int64_t)blockIdx.y * cols + c0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) dst[j] = acc[j];
+}
+
 inline void colsum_geometry(int64_t rows, int64_t cols, int vec, int* gx, int* splits, int* rps) {
     *gx = (int)((cols + 128 * vec - 1) / (128 * vec));
     int64_t s = 2048 / *gx;
@@ -517,6 +577,30 @@ int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t row
     PTJ_CHECK_LAUNCH();
     hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
                        (const float*)ws, splits, (int)cols, (T*)out);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+template <typename T>
+int gelu_bwd_colsum_impl(const void* dy, const void* x, void* dx, void* colsum, void* ws, size_t ws_bytes, int64_t rows,
+                         int64_t cols, hipStream_t st) {
+    constexpr int FV = VecOf<T>::N;
+    const bool vok = (cols % FV == 0) && ptj_aligned16(x) && ptj_aligned16(dy) && ptj_aligned16(dx);
+    const int vec = vok ? FV : 1;
+    int gx, splits, rps;
+    colsum_geometry(rows, cols, vec, &gx, &splits, &rps);
+    const size_t need = (size_t)splits * cols * sizeof(float);
+    if (!ws || ws_bytes < need)
+        return ptj_set_error(PTJ_ERR_WORKSPACE, "gelu_bwd_colsum: workspace %zu < %zu bytes", ws_bytes, need);
+    if (vok)
+        hipLaunchKernelGGL((gelu_bwd_colsum_kernel<T, FV>), dim3(gx, splits), dim3(128), 0, st, (const T*)dy, (const T*)x,
+                           (T*)dx, (float*)ws, rows, (int)cols, rps);
+    else
+        hipLaunchKernelGGL((gelu_bwd_colsum_kernel<T, 1>), dim3(gx, splits), dim3(128), 0, st, (const T*)dy, (const T*)x,
+                           (T*)dx, (float*)ws, rows, (int)cols, rps);
+    PTJ_CHECK_LAUNCH();
+    hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
+                       (const float*)ws, splits, (int)cols, (T*)colsum);
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
 }
@@ -614,7 +698,7 @@ template <typename T>
 int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const void* res, void* dx, void* dgamma,
                        void* dbeta,
                        void* ws, size_t ws_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs, int64_t dxs,
-                       void* drop, int drop_train, int64_t drop_seed, const void* keep, hipStream_t st) {
+                       void* drop, int drop_train, int64_t drop_seed, const void* keep, void* drop_sum, hipStream_t st) {
     RowCfg cfg;
     const bool vok = rows_vec_ok<T>(cols, {dy, x, gamma, dx, res, drop}, {dys, xs, dx ? dxs : 0});
     if (keep != nullptr && !(vok && VecOf<T>::N == 8))
@@ -624,8 +708,11 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
     const int grid = ln_bwd_grid(rows, cfg.tpr);
     const int nparts = grid;
     const bool want_dx = dx != nullptr, want_dgb = dgamma != nullptr;
+    const int np = drop_sum != nullptr ? 3 : 2;
+    if (drop_sum != nullptr && !(want_dgb && drop != nullptr))
+        return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: the column sums of the dropped output need dgamma/dbeta and the dropped output");
     if (want_dgb) {
-        const size_t need = (size_t)nparts * 2 * (size_t)cols * sizeof(float);
+        const size_t need = (size_t)nparts * np * (size_t)cols * sizeof(float);
         if (!ws || ws_bytes < need)
             return ptj_set_error(PTJ_ERR_WORKSPACE, "layernorm_bwd: workspace %zu < %zu bytes", ws_bytes, need);
     }
@@ -633,7 +720,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
     hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
                        dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (const T_*)res, (T_*)dx, \
                        (float*)ws, rows, (int)cols, dys, xs, dxs, (T_*)drop, drop_train, (uint64_t)drop_seed,    \
-                       (const uint8_t*)keep)
+                       (const uint8_t*)keep, np)
 #define LAUNCH(T_, V_, TPR_, IT_)                                     \
     do {                                                              \
         if (want_dx && want_dgb) LAUNCH_F(T_, V_, TPR_, IT_, true, true);   \
@@ -645,8 +732,8 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
 #undef LAUNCH_F
     PTJ_CHECK_LAUNCH();
     if (want_dgb) {
-        hipLaunchKernelGGL((layernorm_bwd_reduce_kernel<T>), dim3((unsigned)((cols + 31) / 32), 2), dim3(RED_THREADS), 0, st,
-                           (const float*)ws, nparts, (int)cols, (T*)dgamma, (T*)dbeta);
+        hipLaunchKernelGGL((layernorm_bwd_reduce_kernel<T>), dim3((unsigned)((cols + 31) / 32), np), dim3(RED_THREADS), 0, st,
+                           (const float*)ws, nparts, (int)cols, (T*)dgamma, (T*)dbeta, (T*)drop_sum);
         PTJ_CHECK_LAUNCH();
     }
     return PTJ_OK;
@@ -766,11 +853,11 @@ int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* 
 size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     // Upper bound over the row configurations the dispatcher can pick.
-    return (size_t)512 * 2 * (size_t)cols * sizeof(float);
+    return (size_t)512 * 3 * (size_t)cols * sizeof(float);
 }
 
 int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, const void* residual, void* dx,
-                              void* dgamma, void* dbeta, void* dropped, int drop_train, int64_t drop_seed,
+                              void* dgamma, void* dbeta, void* dropped, void* dropped_colsum, int drop_train, int64_t drop_seed,
                               const void* keep_bytes, void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys,
                               int64_t xs, int64_t dxs, int dtype, void* stream) {
     PTJ_CHECK_ARG(dy && x, "layernorm_bwd: null dy/x");
@@ -778,22 +865,23 @@ int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, 
     PTJ_CHECK_ARG(!dx || gamma, "layernorm_bwd: dx requested without gamma");
     PTJ_CHECK_ARG(!residual || dx, "layernorm_bwd: residual given without dx");
     PTJ_CHECK_ARG(!dropped || dx, "layernorm_bwd: dropout output requested without dx");
+    PTJ_CHECK_ARG(!dropped_colsum || (dropped && dgamma), "layernorm_bwd: dropped_colsum needs dropped and dgamma/dbeta");
     PTJ_CHECK_ARG((dgamma == nullptr) == (dbeta == nullptr), "layernorm_bwd: dgamma and dbeta must be given together");
     PTJ_CHECK_ARG(rows >= 1 && cols >= 2, "layernorm_bwd: need rows >= 1 and cols >= 2");
     PTJ_CHECK_ARG(dys >= cols && xs >= cols && (!dx || dxs >= cols), "layernorm_bwd: row stride smaller than cols");
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype,
                  (layernorm_bwd_impl<float>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols,
-                                            dys, xs, dxs, dropped, drop_train, drop_seed, keep_bytes, st)),
+                                            dys, xs, dxs, dropped, drop_train, drop_seed, keep_bytes, dropped_colsum, st)),
                  (layernorm_bwd_impl<bf16>(dy, x, gamma, residual, dx, dgamma, dbeta, workspace, workspace_bytes, rows, cols, dys,
-                                           xs, dxs, dropped, drop_train, drop_seed, keep_bytes, st)));
+                                           xs, dxs, dropped, drop_train, drop_seed, keep_bytes, dropped_colsum, st)));
 }
 
 int ptj_layernorm_bwd(const void* dy, const void* x, const void* gamma, const void* residual, void* dx, void* dgamma,
                       void* dbeta,
                       void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t dys, int64_t xs,
                       int64_t dxs, int dtype, void* stream) {
-    return ptj_layernorm_bwd_dropout(dy, x, gamma, residual, dx, dgamma, dbeta, nullptr, 0, 0, nullptr, workspace, workspace_bytes,
+    return ptj_layernorm_bwd_dropout(dy, x, gamma, residual, dx, dgamma, dbeta, nullptr, nullptr, 0, 0, nullptr, workspace, workspace_bytes,
                                      rows, cols, dys, xs, dxs, dtype, stream);
 }
 
@@ -830,6 +918,15 @@ int ptj_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype, 
     PTJ_CHECK_ARG(n >= 0 && (n == 0 || (dy && x && dx)), "gelu_bwd: bad arguments");
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype, (gelu_impl<float>(dy, x, dx, n, true, st)), (gelu_impl<bf16>(dy, x, dx, n, true, st)));
+}
+
+int ptj_gelu_bwd_colsum(const void* dy, const void* x, void* dx, void* colsum, void* workspace, size_t workspace_bytes,
+                        int64_t rows, int64_t cols, int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 31), "gelu_bwd_colsum: bad shape");
+    PTJ_CHECK_ARG(dy && x && dx && colsum, "gelu_bwd_colsum: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (gelu_bwd_colsum_impl<float>(dy, x, dx, colsum, workspace, workspace_bytes, rows, cols, st)),
+                 (gelu_bwd_colsum_impl<bf16>(dy, x, dx, colsum, workspace, workspace_bytes, rows, cols, st)));
 }
 
 int ptj_dropout(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, int train, int64_t seed,

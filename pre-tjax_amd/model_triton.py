@@ -81,6 +81,23 @@ def t_gelu_bkwd2_t(dloss_dx: torch.Tensor, x: torch.Tensor):
     return out.reshape(x.shape)
 
 
+def t_gelu_bkwd2_colsum_t(dloss_dx: torch.Tensor, x: torch.Tensor):
+    """GELU backward plus the column sums of its result in one pass:
+    ``(t_gelu_bkwd2_t(dloss_dx, x), colsum_t(of that))`` -- dx and the gradient of the bias
+    in front of the activation (model_triton.py:296-304, :426)."""
+    require_gpu(dloss_dx, x)
+    assert dloss_dx.shape == x.shape and dloss_dx.dtype == x.dtype
+    dc, xc = _rows2d(dloss_dx).contiguous(), _rows2d(x).contiguous()
+    rows, cols = xc.shape
+    out = torch.empty_like(xc)
+    sums = torch.empty(cols, dtype=xc.dtype, device=xc.device)
+    ws_bytes = lib().ptj_colsum_workspace_bytes(rows, cols)
+    ws = _workspace(ws_bytes, xc.device, "colsum")
+    check(lib().ptj_gelu_bwd_colsum(ptr(dc), ptr(xc), ptr(out), ptr(sums), ptr(ws), ws_bytes, rows, cols,
+                                    dtype_code(xc), stream()), "ptj_gelu_bwd_colsum")
+    return out.reshape(x.shape), sums
+
+
 # ----------------------------------------------------------------------------------
 # dropout  (reference: model_triton.py:1496-1506, :1562-1572)
 # ----------------------------------------------------------------------------------
@@ -151,7 +168,7 @@ def t_layernorm_fwd_t(layer_params, x: torch.Tensor):
     return out.reshape(x.shape)
 
 
-def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None, drop=None):
+def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None, drop=None, drop_sum=False):
     require_gpu(dloss_dx, x)
     d2, x2 = _rows2d(dloss_dx), _rows2d(x)
     assert d2.shape == x2.shape and d2.dtype == x2.dtype
@@ -174,11 +191,18 @@ def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None, dr
         d_train, d_seed = int(bool(drop[0])), int(drop[1] if drop[0] else 0)
         keep = drop[2] if len(drop) > 2 and drop[0] else None
         dropped = torch.empty_like(dx)
+    dsum = None
+    if drop_sum:
+        assert drop is not None and want_p
+        dsum = torch.empty_like(gamma)
     check(lib().ptj_layernorm_bwd_dropout(ptr(d2), ptr(x2), ptr(gamma), ptr(residual), ptr(dx), ptr(dg), ptr(db),
-                                          ptr(dropped), d_train, d_seed, ptr(keep), ptr(ws), ws_bytes, rows, cols, d2.stride(0),
-                                          x2.stride(0), dx.stride(0) if want_dx else 0, dtype_code(x2), stream()),
+                                          ptr(dropped), ptr(dsum), d_train, d_seed, ptr(keep), ptr(ws), ws_bytes, rows,
+                                          cols, d2.stride(0), x2.stride(0), dx.stride(0) if want_dx else 0,
+                                          dtype_code(x2), stream()),
           "ptj_layernorm_bwd")
     dx_out = dx.reshape(dloss_dx.shape) if want_dx else None
+    if drop_sum:
+        return dx_out, dg, db, dropped.reshape(dloss_dx.shape), dsum
     if drop is not None:
         return dx_out, dg, db, dropped.reshape(dloss_dx.shape)
     return dx_out, dg, db
@@ -194,12 +218,18 @@ def t_layernorm_bkwd2_x_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor)
     return dx
 
 
-def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, residual=None, drop=None):
+def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, residual=None, drop=None,
+                      drop_sum=False):
     """dx (+ residual), (dgamma, dbeta) from one read of dy and x (fusion of the two
     reference launches at model_triton.py:2033-2034 and of the residual add at :2036).
     With ``drop=(train, seed[, keep])`` a third result is t_dropout_bkwd2_t(dx, None, train,
     seed) (the dropout backward the block applies next, :2021-2024), written in the same
-    pass; `keep` are the keep bytes recorded by dropout_add_t for that seed, if any."""
+    pass; `keep` are the keep bytes recorded by dropout_add_t for that seed, if any.  With
+    ``drop_sum=True`` a fourth result is colsum_t of that third one (the bias gradient of
+    the linear layer whose output gradient it is, :426)."""
+    if drop_sum:
+        dx, dg, db, dropped, dsum = _layernorm_bwd(dloss_dx, layer_params, x, True, True, residual, drop, True)
+        return dx, (dg, db), dropped, dsum
     if drop is not None:
         dx, dg, db, dropped = _layernorm_bwd(dloss_dx, layer_params, x, True, True, residual, drop)
         return dx, (dg, db), dropped
@@ -439,13 +469,15 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
 
 
 def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_aux=None, dropped_in=None,
-                          drop_out=None):
+                          drop_out=None, db2_in=None, drop_out_sum=False):
     """Backward of one block (model_triton.py:2291-2299 and the sub-block VJPs :2021-2039,
     :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order).
 
     `dropped_in`, if given, is t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2]) already
     computed by the producer of dloss_dx; `drop_out=(train, seed)` asks for the same service
-    for the consumer of dx: the result is then (dx, grads, dropout_bkwd(dx))."""
+    for the consumer of dx: the result is then (dx, grads, dropout_bkwd(dx)).  `db2_in` is
+    colsum_t(dropped_in) if the producer also summed it; `drop_out_sum` appends the column
+    sums of the dropped dx to the result."""
     if not train:
         p_gen_aux = [0, 0, 0]
     ln1g, ln1b, wqkv, wo, ln2g, ln2b, w1, b1, w2, b2 = layer_params
@@ -456,11 +488,10 @@ def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_
     B = N // T
     # ---- sub-block 2: x_out = x_mid + dropout(ffn(ln2(x_mid)))
     d = dropped_in if dropped_in is not None else t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2])
-    db2 = colsum_t(d)
+    db2 = db2_in if (db2_in is not None and dropped_in is not None) else colsum_t(d)
     dw2 = matmul_t(d.t(), g1)                                           # [D,F]
     dg1 = matmul_t(d, w2)                                               # [N,F]
-    df1 = t_gelu_bkwd2_t(dg1, f1)
-    db1 = colsum_t(df1)
+    df1, db1 = t_gelu_bkwd2_colsum_t(dg1, f1)
     dw1 = matmul_t(df1.t(), h2)                                         # [F,D]
     dh2 = matmul_t(df1, w1)                                             # [N,D]
     dx_mid, (dln2g, dln2b), d = layernorm_bkwd2_t(dh2, (ln2g, ln2b), x_mid, residual=dloss_dx,
@@ -478,12 +509,17 @@ def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_
     attn_bwd_t(do4, q, k, v, o4, ms, ls, mask, train, p_gen_aux[0], out=outs)
     dwqkv = matmul_t(dqkv.t(), h1).view(H, 3, dh, D)                    # [H*3*dh, D]
     dh1 = matmul_t(dqkv, wqkv.view(H * 3 * dh, D))                      # [N,D]
-    grads = None
-    if drop_out is not None:
+    dsum = None
+    if drop_out is not None and drop_out_sum:
+        dx_in, (dln1g, dln1b), dropped, dsum = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid,
+                                                                 drop=drop_out, drop_sum=True)
+    elif drop_out is not None:
         dx_in, (dln1g, dln1b), dropped = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid, drop=drop_out)
     else:
         dx_in, (dln1g, dln1b) = layernorm_bkwd2_t(dh1, (ln1g, ln1b), x_in, residual=dx_mid)
     grads = [dln1g, dln1b, dwqkv, dwo, dln2g, dln2b, dw1, db1, dw2, db2]
+    if drop_out is not None and drop_out_sum:
+        return dx_in, grads, dropped, dsum
     if drop_out is not None:
         return dx_in, grads, dropped
     return dx_in, grads
@@ -543,18 +579,22 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
     # so each LayerNorm backward also writes the dropped copy its consumer needs: the final
     # norm for the last block's FFN dropout (seed 3L), block i's first norm for block i-1's
     # FFN dropout (seed 3i) or, for block 0, for the embedding dropout (seed 0).
+    dsum = None                                                         # colsum_t(dropped): block i's db2
     if L > 0:
-        dx, (dlnfg, dlnfb), dropped = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D),
-                                                       drop=(train, p_gen_aux[3 * L], layer_acts[L - 1][-1]))
+        dx, (dlnfg, dlnfb), dropped, dsum = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D),
+                                                             drop=(train, p_gen_aux[3 * L], layer_acts[L - 1][-1]),
+                                                             drop_sum=True)
     else:
         dx, (dlnfg, dlnfb), dropped = layernorm_bkwd2_t(dh, params[-1], x_last.reshape(N, D),
                                                        drop=(train, p_gen_aux[0]))
     layer_grads = [None] * L
     for i in reversed(range(L)):
-        dx, layer_grads[i], dropped = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train,
-                                                            p_gen_aux[1 + 3 * i:4 + 3 * i], dropped_in=dropped,
-                                                            drop_out=(train, p_gen_aux[3 * i],
-                                                                      layer_acts[i - 1][-1] if i > 0 else None))
+        res = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i],
+                                    dropped_in=dropped, db2_in=dsum,
+                                    drop_out=(train, p_gen_aux[3 * i], layer_acts[i - 1][-1] if i > 0 else None),
+                                    drop_out_sum=i > 0)
+        dx, layer_grads[i], dropped = res[:3]
+        dsum = res[3] if i > 0 else None
     d = dropped                                                         # [N,D] = dropout_bkwd(dx, seed 0)
     # positional table: sum over the batch (model_triton.py:2518 with indices = arange(T))
     dpos = torch.zeros_like(params[1][0])

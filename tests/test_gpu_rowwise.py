@@ -70,6 +70,24 @@ def test_gelu(mt, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(16384, 3072), (1000, 768), (37, 101), (1, 8), (2, 3, 64)])
+def test_gelu_bwd_with_colsum_matches_separate_calls(mt, dtype, shape):
+    """The fused entry point writes exactly the dx of t_gelu_bkwd2_t and the column sums of
+    that stored dx (compared with an fp64 sum of the rounded values)."""
+    g = gen(11)
+    x, dy = randn(g, *shape, dtype=dtype, std=2.0).to(DEV), randn(g, *shape, dtype=dtype).to(DEV)
+    dx, sums = mt.t_gelu_bkwd2_colsum_t(dy, x)
+    want = mt.t_gelu_bkwd2_t(dy, x)
+    assert dx.shape == x.shape and torch.equal(dx, want)
+    rows = x.numel() // shape[-1]
+    ref = f64(want).reshape(rows, shape[-1]).sum(0)
+    tol = (3e-6 if dtype == torch.float32 else 8e-3) * max(1.0, rows ** 0.5)
+    assert (f64(sums) - ref).abs().max().item() <= tol + (0 if dtype == torch.float32 else 1e-2 * ref.abs().max().item())
+    dx2, sums2 = mt.t_gelu_bkwd2_colsum_t(dy, x)
+    assert torch.equal(sums, sums2) and torch.equal(dx, dx2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape,seed", [((8192, 768), 42), ((2, 3, 768), 7), ((5, 100), 123456), ((3, 1001), 999999),
                                         ((4, 8), (1 << 32) + 5)])
 def test_dropout_mask_bit_exact(mt, dtype, shape, seed):
@@ -158,3 +176,11 @@ def test_layernorm_bwd_with_dropout_output_matches_separate_calls(mt, dtype, sha
             assert torch.equal(got2, want)
         else:
             assert not (train and dtype == torch.bfloat16 and shape[1] % 8 == 0)
+        # and with the column sums of the dropped output (a bias gradient) from the same pass
+        dx3, (dg3, db3), got3, sums = mt.layernorm_bkwd2_t(dy, (gamma, beta), x, residual=res, drop=(train, 4242),
+                                                           drop_sum=True)
+        assert torch.equal(dx3, dx0) and torch.equal(dg3, dg0) and torch.equal(db3, db0) and torch.equal(got3, want)
+        ref = f64(want).sum(0)
+        rows = shape[0]
+        tol = (3e-6 if dtype == torch.float32 else 8e-3) * max(1.0, rows ** 0.5)
+        assert (f64(sums) - ref).abs().max().item() <= tol + (0 if dtype == torch.float32 else 1e-2 * ref.abs().max().item())
