@@ -122,6 +122,24 @@ int ptj_dropout_add(const void* x, const void* res, void* y, int64_t rows, int64
 int ptj_dropout_add_keep(const void* x, const void* res, void* y, void* keep_bytes,
                          int64_t rows, int64_t cols, int train, int64_t seed, int dtype, void* stream);
 
+/* Embedding forward: out[i, :] = dropout(round(wemb[tokens[i], :] * scale) + pos[i mod seq, :])
+ * for i < n, with the mask of ptj_dropout(train, seed) on [n, dim] -- t_embed_fwd
+ * (model_triton.py:166-167), the position add and the embedding dropout of
+ * t_gpt2_tlayers_fwd3_t (model_triton.py:2334-2351) in one pass.  Token ids must lie in
+ * [0, vocab). */
+int ptj_embed_fwd(const void* wemb, const void* pos, const int64_t* tokens, void* out,
+                  int64_t n, int64_t dim, int64_t seq, int64_t vocab, float scale,
+                  int train, int64_t seed, int dtype, void* stream);
+
+/* Embedding backward, in place on the table gradient:
+ * dwemb[t, :] += scale * sum_{i: tokens[i] = t} d[i, :] -- the scatter-add of
+ * t_embed_bkwd (model_triton.py:2489-2521) accumulated onto the tied LM-head gradient
+ * (:2591).  `sorted_tokens` are the n token ids in ascending (stable) order and `order`
+ * the permutation that sorts them (sorted_tokens[j] = tokens[order[j]]); every run of equal
+ * ids is summed in that order in fp32, so the result is deterministic. */
+int ptj_embed_bwd(const void* d, const int64_t* sorted_tokens, const int64_t* order, void* dwemb,
+                  int64_t n, int64_t dim, int64_t vocab, float scale, int dtype, void* stream);
+
 /* Row-wise log-softmax forward / backward (dx = dy - softmax(x)*sum(dy)).
  * Replace t_log_softmax_fwd_k/_t (model_triton.py:30-72) and
  * t_log_softmax_bkwd2_k/_t (:122-164). */

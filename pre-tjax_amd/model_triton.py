@@ -441,6 +441,35 @@ def t_embed_fwd(layer_params, x):
     return layer_params[0][x] * math.sqrt(layer_params[0].shape[1])
 
 
+def embed_pos_dropout_t(wemb, pos, y, train=True, p_gen_aux=None):
+    """dropout(t_embed_fwd((wemb,), y) + pos[:T]) in one pass: y int [B,T] -> [B,T,D]
+    (the first three steps of model_triton.py:2334-2351)."""
+    require_gpu(wemb, pos, y)
+    B, T = y.shape
+    V, D = wemb.shape
+    assert pos.shape[0] >= T and pos.shape[1] == D and pos.dtype == wemb.dtype
+    wc, pc = wemb.contiguous(), pos.contiguous()
+    tok = y.reshape(-1).to(torch.int64).contiguous()
+    out = torch.empty((B, T, D), dtype=wemb.dtype, device=wemb.device)
+    check(lib().ptj_embed_fwd(ptr(wc), ptr(pc), ptr(tok), ptr(out), B * T, D, T, V, math.sqrt(D), int(bool(train)),
+                              int(p_gen_aux if train else 0), dtype_code(wc), stream()), "ptj_embed_fwd")
+    return out
+
+
+def embed_bkwd_add_t(dwemb, d, y):
+    """dwemb[tok] += sqrt(D) * (sum of the rows of d [N,D] whose token is tok), in place and
+    deterministic (model_triton.py:2489-2521 scatter-add, accumulated onto the tied LM-head
+    gradient as at :2591)."""
+    require_gpu(dwemb, d, y)
+    V, D = dwemb.shape
+    assert dwemb.is_contiguous() and d.dtype == dwemb.dtype
+    d2 = d.reshape(-1, D).contiguous()
+    stok, order = torch.sort(y.reshape(-1).to(torch.int64), stable=True)
+    check(lib().ptj_embed_bwd(ptr(d2), ptr(stok), ptr(order), ptr(dwemb), d2.shape[0], D, V, math.sqrt(D),
+                              dtype_code(dwemb), stream()), "ptj_embed_bwd")
+    return dwemb
+
+
 def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
     """One block (model_triton.py:2214-2223).  y [B,T,D] -> (y_out, acts)."""
     if not train:
@@ -532,8 +561,7 @@ def t_gpt2_tlayers_fwd3_t(params, y, mask, indices, train=True, p_gen_aux=None):
         p_gen_aux = [0] * (1 + 3 * L)
     T = y.shape[1]
     assert T <= params[1][0].shape[0], "sequence longer than the positional table"
-    x = t_embed_fwd(params[0], y) + params[1][0][:T]
-    x = t_dropout_fwd_t(x, train, p_gen_aux[0])
+    x = embed_pos_dropout_t(params[0][0], params[1][0], y, train, p_gen_aux[0])
     layer_acts = []
     for i, lp in enumerate(params[2:-1]):
         x, a = t_gpt2_tlayer_fwd3_t(lp, x, mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i])
@@ -600,7 +628,5 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
     dpos = torch.zeros_like(params[1][0])
     dpos[:T] = colsum_t(d.view(B, T * D)).view(T, D)
     # embedding: scatter-add rows by token id, times sqrt(D); tied with the LM head (:2591)
-    demb = torch.zeros((V, D), dtype=torch.float32, device=d.device)
-    demb.index_add_(0, y.reshape(-1).to(torch.int64), d.to(torch.float32))
-    dwemb = (dwemb.to(torch.float32) + demb * math.sqrt(D)).to(wemb.dtype)
+    dwemb = embed_bkwd_add_t(dwemb, d, y)
     return [[dwemb, dbemb], [dpos]] + layer_grads + [[dlnfg, dlnfb]]
