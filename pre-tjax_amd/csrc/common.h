@@ -64,15 +64,30 @@ __device__ __forceinline__ void store_vec(T* __restrict__ p, const float (&in)[N
 }
 
 // ---- wavefront (64 lanes) reductions --------------------------------------------
+// All 64 lanes must be active.  Lanes are combined inside each row of 16 with DPP lane
+// permutations (quad swaps, then row rotations by 4 and 8: no LDS crossbar round trips),
+// and the four row results are read out and combined in row order, so every lane returns
+// the same value and the order of the additions is fixed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += dpp_move<0x124>(v);   // row_ror 4
+    v += dpp_move<0x128>(v);   // row_ror 8
+    return ((lane_value(v, 0) + lane_value(v, 16)) + lane_value(v, 32)) + lane_value(v, 48);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x124>(v));
+    v = fmaxf(v, dpp_move<0x128>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
 // Reduction over the TPR threads that share one row.  TPR == 64: one wave, no LDS.

@@ -36,6 +36,22 @@ struct RowRegs {
     }
 };
 
+// One row in storage type (ITERS 16-byte vectors per thread), for operands that are used
+// once and late: they wait in a quarter (bf16) of the registers of their float form.
+template <typename T, int VEC, int TPR, int ITERS>
+struct RawRow {
+    Pack<T, VEC> p[ITERS];
+    __device__ __forceinline__ void load(const T* __restrict__ row, int nvec, int t) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int vi = t + it * TPR;
+            const int vc = vi < nvec ? vi : nvec - 1;   // lanes past the row re-read its last vector
+            p[it] = *reinterpret_cast<const Pack<T, VEC>*>(row + (int64_t)vc * VEC);
+        }
+    }
+    __device__ __forceinline__ float get(int it, int j) const { return to_f32(p[it].v[j]); }
+};
+
 template <int TPR> struct RowGeom {
     static constexpr int BLOCK = TPR == 64 ? 256 : TPR;
     static constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
@@ -93,17 +109,29 @@ __global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_fwd_kernel(
 // Partials layout: part[p][0][cols] = sum dy*xhat, part[p][1][cols] = sum dy over the
 // rows handled by row-slot p (p = blockIdx.x*RPB + sub).
 // ---------------------------------------------------------------------------------
+#ifndef PTJ_LN_BLOCK
+#define PTJ_LN_BLOCK 512
+#endif
+#ifndef PTJ_LN_MINW
+#define PTJ_LN_MINW 4
+#endif
 template <int TPR> struct LnBwdGeom {
-    static constexpr int BLOCK = TPR == 64 ? 512 : TPR;
+    static constexpr int BLOCK = TPR == 64 ? PTJ_LN_BLOCK : TPR;
     static constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
 };
 constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave holds (bf16, ITERS 4)
 
-template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB>
-__global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
+// DROP selects the code for the second (dropout) output at compile time, which keeps the
+// Philox generator out of the register budget of the common variants: 0 = no second
+// output, 1 = mask read from recorded keep bytes, 2 = mask recomputed (or eval scaling).
+template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB, int DROP>
+__global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK, (TPR == 64 && ITERS <= 3 && DROP != 2) ? PTJ_LN_MINW : 2) void layernorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
     T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs,
-    T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep, int np) {
+    T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep, int np,
+    int has_res, int64_t ress) {
+    // res is always a readable row source (the host passes dy when there is no residual), so
+    // that its load is unconditional; has_res says whether it is added.
     // np: partial sums per workgroup and column: dgamma, dbeta and, with np == 3, the
     // column sums of the `drop` output
     __shared__ float smem[16];
@@ -111,8 +139,8 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const int t = threadIdx.x % TPR;
     const int sub = threadIdx.x / TPR;
     const int nvec = cols / VEC;
-    RowRegs<T, VEC, TPR, ITERS> g;
-    if constexpr (DX) g.load(gamma, nvec, t, 0.f);
+    RawRow<T, VEC, TPR, ITERS> g;
+    if constexpr (DX) g.load(gamma, nvec, t);
     float acc_g[ITERS][VEC], acc_b[ITERS][VEC], acc_d[ITERS][VEC];
     if constexpr (DGB) {
 #pragma unroll
@@ -125,14 +153,25 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
     const float n_adj = (float)cols * inv_nm1;
     // Every thread of a >64-thread row group must take the same trip count because
     // row_reduce synchronises the block; with RPB == 1 all threads share `row`.
+#pragma unroll 1
     for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
-        RowRegs<T, VEC, TPR, ITERS> r, d, rr;
+        RowRegs<T, VEC, TPR, ITERS> r, d;
+        RawRow<T, VEC, TPR, ITERS> rr;
         r.load(x + row * xs, nvec, t, 0.f);
         d.load(dy + row * dys, nvec, t, 0.f);
         if constexpr (DX) {
-            // residual row, in flight under the reductions; without a residual the (cached)
-            // dy row is re-read and ignored, which keeps the load out of a branch
-            rr.load(res != nullptr ? res + row * (int64_t)cols : dy + row * dys, nvec, t, 0.f);
+            // residual row, in flight under the reductions
+            rr.load(res + row * ress, nvec, t);
+        }
+        uint32_t kbits[ITERS];
+        if constexpr (DROP == 1) {
+            // keep bytes of this row (one per vector), fetched with the row instead of after it
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int vi = t + it * TPR;
+                const int c0 = (vi < nvec ? vi : nvec - 1) * VEC;          // one keep byte per 8 columns
+                kbits[it] = (uint32_t)keep[row * (int64_t)(cols >> 3) + (c0 >> 3)] >> (c0 & 7);
+            }
         }
         float s = 0.f;
 #pragma unroll
@@ -165,7 +204,7 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                     acc_b[it][j] += d.v[it][j];
                 }
                 if constexpr (DX) {
-                    const float gg = d.v[it][j] * g.v[it][j];
+                    const float gg = d.v[it][j] * g.get(it, j);
                     d.v[it][j] = gg;
                     sg += gg;
                     sgx += gg * xh;
@@ -178,16 +217,16 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
             for (int it = 0; it < ITERS; ++it)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) d.v[it][j] = (d.v[it][j] - mg - r.v[it][j] * mgx) * rstd;
-            if (res != nullptr) {
+            if (has_res) {
                 // residual branch: the sum is formed from the storage-rounded LayerNorm gradient,
                 // as two separate passes would
 #pragma unroll
                 for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) d.v[it][j] = rr.v[it][j] + to_f32(from_f32<T>(d.v[it][j]));
+                    for (int j = 0; j < VEC; ++j) d.v[it][j] = rr.get(it, j) + to_f32(from_f32<T>(d.v[it][j]));
             }
             d.store(dx + row * dxs, nvec, t);
-            if (drop != nullptr) {
+            if constexpr (DROP != 0) {
                 // second output: dropout applied to the stored (rounded) dx, i.e. the backward
                 // of the dropout that feeds this residual stream -- saves a pass over dx
                 const uint64_t sd = drop_seed + (uint64_t)row;
@@ -198,12 +237,14 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK) void layernorm_bwd_kernel(
                     // keep bits of this vector: recorded by the forward dropout (one byte per
                     // 8 columns) when available, else recomputed
                     uint32_t bits = 0;
-                    if (VEC == 8 && keep != nullptr) {
-                        bits = keep[row * (int64_t)nvec + (vi < nvec ? vi : nvec - 1)];
-                    } else if (drop_train) {
+                    if constexpr (DROP == 1) {
+                        bits = kbits[it];
+                    } else {
+                        if (drop_train) {
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j)
-                            bits |= philox_keep((uint32_t)(vi * VEC + j), k0, k1) ? (1u << j) : 0u;
+                            for (int j = 0; j < VEC; ++j)
+                                bits |= philox_keep((uint32_t)(vi * VEC + j), k0, k1) ? (1u << j) : 0u;
+                        }
                     }
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
@@ -688,9 +729,9 @@ int layernorm_fwd_impl(const void* x, const void* gamma, const void* beta, void*
 
 // Grid of the backward kernel = number of dgamma/dbeta partials (one per workgroup).
 inline int ln_bwd_grid(int64_t rows, int tpr) {
-    const int rpb = tpr == 64 ? 8 : 1;
+    const int rpb = tpr == 64 ? LnBwdGeom<64>::ROWS_PER_BLOCK : 1;
     const int64_t need = (rows + rpb - 1) / rpb;
-    const int64_t cap = 512;  // 2 workgroups per CU: bounds the partials to 512 rows of 2*cols floats
+    const int64_t cap = tpr == 64 ? 512 * (512 / LnBwdGeom<64>::BLOCK) : 512;  // bounds the partials
     return (int)(need < cap ? need : cap);
 }
 
@@ -709,6 +750,8 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
     const int nparts = grid;
     const bool want_dx = dx != nullptr, want_dgb = dgamma != nullptr;
     const int np = drop_sum != nullptr ? 3 : 2;
+    // keep bytes are read by the variant with dgamma/dbeta only; elsewhere the mask is recomputed
+    const int drop_mode = drop == nullptr ? 0 : (keep != nullptr && want_dgb && drop_train) ? 1 : 2;
     if (drop_sum != nullptr && !(want_dgb && drop != nullptr))
         return ptj_set_error(PTJ_ERR_INVALID, "layernorm_bwd: the column sums of the dropped output need dgamma/dbeta and the dropped output");
     if (want_dgb) {
@@ -716,18 +759,33 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
         if (!ws || ws_bytes < need)
             return ptj_set_error(PTJ_ERR_WORKSPACE, "layernorm_bwd: workspace %zu < %zu bytes", ws_bytes, need);
     }
-#define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_)                                                                   \
-    hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_>), dim3(grid),                         \
-                       dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma, (const T_*)res, (T_*)dx, \
+#define LAUNCH_F(T_, V_, TPR_, IT_, DX_, DGB_, DROP_)                                                            \
+    hipLaunchKernelGGL((layernorm_bwd_kernel<T_, V_, TPR_, IT_, DX_, DGB_, DROP_>), dim3(grid),                  \
+                       dim3(LnBwdGeom<TPR_>::BLOCK), 0, st, (const T_*)dy, (const T_*)x, (const T_*)gamma,       \
+                       (const T_*)(res ? res : dy), (T_*)dx,                                                     \
                        (float*)ws, rows, (int)cols, dys, xs, dxs, (T_*)drop, drop_train, (uint64_t)drop_seed,    \
-                       (const uint8_t*)keep, np)
+                       (const uint8_t*)keep, np, res ? 1 : 0, res ? cols : dys)
 #define LAUNCH(T_, V_, TPR_, IT_)                                     \
     do {                                                              \
-        if (want_dx && want_dgb) LAUNCH_F(T_, V_, TPR_, IT_, true, true);   \
-        else if (want_dx) LAUNCH_F(T_, V_, TPR_, IT_, true, false);   \
-        else LAUNCH_F(T_, V_, TPR_, IT_, false, true);                \
+        if (want_dx && want_dgb) {                                    \
+            if (drop_mode == 0) LAUNCH_F(T_, V_, TPR_, IT_, true, true, 0);        \
+            else if (drop_mode == 1) LAUNCH_F(T_, V_, TPR_, IT_, true, true, 1);   \
+            else LAUNCH_F(T_, V_, TPR_, IT_, true, true, 2);          \
+        } else if (want_dx) {                                         \
+            if (drop_mode == 0) LAUNCH_F(T_, V_, TPR_, IT_, true, false, 0);       \
+            else LAUNCH_F(T_, V_, TPR_, IT_, true, false, 2);         \
+        } else LAUNCH_F(T_, V_, TPR_, IT_, false, true, 0);           \
     } while (0)
-    ROW_DISPATCH(T, cfg, LAUNCH);
+    // 2-byte rows of 513..768 columns: three 8-byte vectors per lane keep all 64 lanes busy and
+    // need a quarter fewer registers than two 16-byte vectors (one more wave per SIMD)
+    bool launched = false;
+    if constexpr (sizeof(T) == 2) {
+        if (cfg.vec == 8 && cfg.tpr == 64 && cols > 512 && cols <= 768) {
+            LAUNCH(T, 4, 64, 3);
+            launched = true;
+        }
+    }
+    if (!launched) ROW_DISPATCH(T, cfg, LAUNCH);
 #undef LAUNCH
 #undef LAUNCH_F
     PTJ_CHECK_LAUNCH();
@@ -853,7 +911,7 @@ int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* 
 size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     // Upper bound over the row configurations the dispatcher can pick.
-    return (size_t)512 * 3 * (size_t)cols * sizeof(float);
+    return (size_t)(512 * (512 / LnBwdGeom<64>::BLOCK)) * 3 * (size_t)cols * sizeof(float);
 }
 
 int ptj_layernorm_bwd_dropout(const void* dy, const void* x, const void* gamma, const void* residual, void* dx,
