@@ -140,6 +140,15 @@ int ptj_embed_fwd(const void* wemb, const void* pos, const int64_t* tokens, void
 int ptj_embed_bwd(const void* d, const int64_t* sorted_tokens, const int64_t* order, void* dwemb,
                   int64_t n, int64_t dim, int64_t vocab, float scale, int dtype, void* stream);
 
+/* ptj_dropout_add[_keep] followed by ptj_layernorm_fwd on its result, in one pass:
+ * y = res + dropout(x), h = layernorm(y) with the values of y as stored -- the residual
+ * update of one sub-block and the normalisation that opens the next one
+ * (model_triton.py:1898 / :2069 then :1625-1637).  All tensors contiguous [rows, cols];
+ * `keep_bytes` (nullable) as in ptj_dropout_add_keep.  Bit-identical to the two calls. */
+int ptj_dropout_add_layernorm(const void* x, const void* res, const void* gamma, const void* beta,
+                              void* y, void* h, void* keep_bytes, int64_t rows, int64_t cols,
+                              int train, int64_t seed, int dtype, void* stream);
+
 /* Row-wise log-softmax forward / backward (dx = dy - softmax(x)*sum(dy)).
  * Replace t_log_softmax_fwd_k/_t (model_triton.py:30-72) and
  * t_log_softmax_bkwd2_k/_t (:122-164). */

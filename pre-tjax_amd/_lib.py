@@ -36,6 +36,7 @@ SIGNATURES = {
     "ptj_dropout_add_keep": (_int, [_p, _p, _p, _p, _i64, _i64, _int, _i64, _int, _p]),
     "ptj_embed_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _c.c_float, _int, _i64, _int, _p]),
     "ptj_embed_bwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _c.c_float, _int, _p]),
+    "ptj_dropout_add_layernorm": (_int, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _int, _i64, _int, _p]),
     "ptj_log_softmax_fwd": (_int, [_p, _p, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_log_softmax_bwd": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_ce_workspace_bytes": (_sz, [_i64]),

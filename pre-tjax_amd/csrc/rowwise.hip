@@ -105,6 +105,100 @@ __global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void layernorm_fwd_kernel(
 }
 
 // ---------------------------------------------------------------------------------
+// Residual update fused with the LayerNorm that consumes it, one row per wave / workgroup:
+//   y = res + dropout(x)    exactly as dropout_kernel<ADD> (keep bytes recorded on request)
+//   h = layernorm(y)        exactly as layernorm_fwd_kernel on the stored y
+// A row's Philox key is uniform over its wave, so the key schedule runs on the scalar unit
+// and y is never re-read.
+// ---------------------------------------------------------------------------------
+template <typename T, int VEC, int TPR, int ITERS>
+__global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void dropout_add_layernorm_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma, const T* __restrict__ beta,
+    T* __restrict__ y, T* __restrict__ h, uint8_t* __restrict__ keep_out, int64_t rows, int cols, int train,
+    uint64_t seed) {
+    __shared__ float smem[16];
+    constexpr int RPB = RowGeom<TPR>::ROWS_PER_BLOCK;
+    const int t = threadIdx.x % TPR;
+    const int sub = threadIdx.x / TPR;
+    const int nvec = cols / VEC;
+    RawRow<T, VEC, TPR, ITERS> g, b;
+    g.load(gamma, nvec, t);
+    b.load(beta, nvec, t);
+    const float inv_n = 1.0f / (float)cols;
+    const float inv_nm1 = 1.0f / (float)(cols - 1);
+    for (int64_t row = (int64_t)blockIdx.x * RPB + sub; row < rows; row += (int64_t)gridDim.x * RPB) {
+        RowRegs<T, VEC, TPR, ITERS> r;
+        RawRow<T, VEC, TPR, ITERS> rr;
+        r.load(x + row * (int64_t)cols, nvec, t, 0.f);
+        rr.load(res + row * (int64_t)cols, nvec, t);
+        const uint64_t sd = seed + (uint64_t)row;
+        // the row, and so the key, is the same for all lanes of the wave
+        const uint32_t k0 = __builtin_amdgcn_readfirstlane((uint32_t)sd);
+        const uint32_t k1 = __builtin_amdgcn_readfirstlane((uint32_t)(sd >> 32));
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int vi = t + it * TPR;
+            const bool valid = vi < nvec;
+            if (train) {
+                uint32_t bits = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const bool keep = philox_keep((uint32_t)(vi * VEC + j), k0, k1);
+                    r.v[it][j] = keep ? r.v[it][j] : 0.f;
+                    bits |= keep ? (1u << j) : 0u;
+                }
+                if constexpr (sizeof(T) == 2 && (VEC == 8 || VEC == 4)) {
+                    if (keep_out != nullptr) {   // one byte per 8 columns
+                        if constexpr (VEC == 8) {
+                            if (valid) keep_out[row * (int64_t)(cols >> 3) + vi] = (uint8_t)bits;
+                        } else {
+                            // lanes 2i and 2i+1 hold the two halves of a byte
+                            const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)bits, 0xB1, 0xf, 0xf, false);
+                            if (valid && (vi & 1) == 0)
+                                keep_out[row * (int64_t)(cols >> 3) + (vi >> 1)] = (uint8_t)(bits | (other << 4));
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) r.v[it][j] *= 0.9f;
+            }
+            // dropout(x) is rounded to the storage type before the add, the sum again on store
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float v = rr.get(it, j) + to_f32(from_f32<T>(r.v[it][j]));
+                r.v[it][j] = valid ? to_f32(from_f32<T>(v)) : 0.f;
+            }
+        }
+        r.store(y + row * (int64_t)cols, nvec, t);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += r.v[it][j];
+        const float mu = row_reduce<TPR, false>(s, smem) * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const bool valid = (t + it * TPR) < nvec;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float d = valid ? r.v[it][j] - mu : 0.f;
+                r.v[it][j] = d;
+                q += d * d;
+            }
+        }
+        const float var = row_reduce<TPR, false>(q, smem) * inv_nm1;
+        const float rstd = 1.0f / sqrtf(var);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[it][j] = g.get(it, j) * (r.v[it][j] * rstd) + b.get(it, j);
+        r.store(h + row * (int64_t)cols, nvec, t);
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // LayerNorm backward: dx and/or per-block partial sums of dgamma, dbeta.
 // Partials layout: part[p][0][cols] = sum dy*xhat, part[p][1][cols] = sum dy over the
 // rows handled by row-slot p (p = blockIdx.x*RPB + sub).
@@ -721,7 +815,45 @@ int layernorm_fwd_impl(const void* x, const void* gamma, const void* beta, void*
 #define LAUNCH(T_, V_, TPR_, IT_)                                                                           \
     hipLaunchKernelGGL((layernorm_fwd_kernel<T_, V_, TPR_, IT_>), dim3(grid), dim3(RowGeom<TPR_>::BLOCK), 0, st, \
                        (const T_*)x, (const T_*)gamma, (const T_*)beta, (T_*)y, rows, (int)cols, xs, ys)
-    ROW_DISPATCH(T, cfg, LAUNCH);
+    // 2-byte rows of 513..768 columns: three 8-byte vectors per lane keep all 64 lanes busy
+    // (the same layout, and so the same summation order, as the fused residual + norm kernel)
+    bool launched = false;
+    if constexpr (sizeof(T) == 2) {
+        if (cfg.vec == 8 && cfg.tpr == 64 && cols > 512 && cols <= 768) {
+            LAUNCH(T, 4, 64, 3);
+            launched = true;
+        }
+    }
+    if (!launched) ROW_DISPATCH(T, cfg, LAUNCH);
+#undef LAUNCH
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+template <typename T>
+int dropout_add_layernorm_impl(const void* x, const void* res, const void* gamma, const void* beta, void* y, void* h,
+                               void* keep, int64_t rows, int64_t cols, int train, int64_t seed, hipStream_t st) {
+    RowCfg cfg;
+    const bool vok = rows_vec_ok<T>(cols, {x, res, gamma, beta, y, h}, {});
+    if (keep != nullptr && !(vok && VecOf<T>::N == 8))
+        return ptj_set_error(PTJ_ERR_INVALID, "dropout_add_layernorm: keep bytes need 2-byte elements, cols %% 8 == 0 and 16-byte aligned rows");
+    if (!pick_row_cfg(cols, VecOf<T>::N, vok, &cfg))
+        return ptj_set_error(PTJ_ERR_INVALID, "dropout_add_layernorm: cols=%lld too large for the register-resident row kernel",
+                             (long long)cols);
+    const int grid = row_grid(rows, cfg.tpr);
+#define LAUNCH(T_, V_, TPR_, IT_)                                                                                  \
+    hipLaunchKernelGGL((dropout_add_layernorm_kernel<T_, V_, TPR_, IT_>), dim3(grid), dim3(RowGeom<TPR_>::BLOCK), 0, st, \
+                       (const T_*)x, (const T_*)res, (const T_*)gamma, (const T_*)beta, (T_*)y, (T_*)h, (uint8_t*)keep, \
+                       rows, (int)cols, train, (uint64_t)seed)
+    // 2-byte rows of 513..768 columns: three 8-byte vectors per lane keep all 64 lanes busy
+    bool launched = false;
+    if constexpr (sizeof(T) == 2) {
+        if (cfg.vec == 8 && cfg.tpr == 64 && cols > 512 && cols <= 768) {
+            LAUNCH(T, 4, 64, 3);
+            launched = true;
+        }
+    }
+    if (!launched) ROW_DISPATCH(T, cfg, LAUNCH);
 #undef LAUNCH
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
@@ -906,6 +1038,17 @@ int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* 
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype, (layernorm_fwd_impl<float>(x, gamma, beta, y, rows, cols, xs, ys, st)),
                  (layernorm_fwd_impl<bf16>(x, gamma, beta, y, rows, cols, xs, ys, st)));
+}
+
+int ptj_dropout_add_layernorm(const void* x, const void* res, const void* gamma, const void* beta, void* y, void* h,
+                              void* keep_bytes, int64_t rows, int64_t cols, int train, int64_t seed, int dtype,
+                              void* stream) {
+    PTJ_CHECK_ARG(rows >= 0 && cols >= 2, "dropout_add_layernorm: need rows >= 0 and cols >= 2");
+    if (rows == 0) return PTJ_OK;
+    PTJ_CHECK_ARG(x && res && gamma && beta && y && h, "dropout_add_layernorm: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    DTYPE_SWITCH(dtype, (dropout_add_layernorm_impl<float>(x, res, gamma, beta, y, h, keep_bytes, rows, cols, train, seed, st)),
+                 (dropout_add_layernorm_impl<bf16>(x, res, gamma, beta, y, h, keep_bytes, rows, cols, train, seed, st)));
 }
 
 size_t ptj_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) {

@@ -168,6 +168,30 @@ def t_layernorm_fwd_t(layer_params, x: torch.Tensor):
     return out.reshape(x.shape)
 
 
+def dropout_add_layernorm_t(x: torch.Tensor, residual: torch.Tensor, layer_params, train=True, p_gen_aux=None,
+                            want_keep=False):
+    """``y = residual + dropout(x)`` and ``h = layernorm(y)`` in one pass: dropout_add_t followed
+    by t_layernorm_fwd_t without re-reading y (model_triton.py:1898 / :2069 then :1625-1637).
+    Returns (y, h, keep) with `keep` as in dropout_add_t (None unless recorded)."""
+    require_gpu(x, residual)
+    assert x.shape == residual.shape and x.dtype == residual.dtype
+    if not train:
+        p_gen_aux = 0
+    xc, rc = x.contiguous(), residual.contiguous()
+    gamma, beta = layer_params[0].contiguous(), layer_params[1].contiguous()
+    cols = xc.shape[-1]
+    rows = xc.numel() // cols
+    assert gamma.dtype == xc.dtype and beta.dtype == xc.dtype and gamma.numel() == cols
+    y, h = torch.empty_like(xc), torch.empty_like(xc)
+    keep = None
+    if want_keep and train and _keep_bytes_ok(xc) and _keep_bytes_ok(rc):
+        keep = torch.empty(rows * (cols // 8), dtype=torch.uint8, device=xc.device)
+    check(lib().ptj_dropout_add_layernorm(ptr(xc), ptr(rc), ptr(gamma), ptr(beta), ptr(y), ptr(h), ptr(keep), rows, cols,
+                                          int(bool(train)), int(p_gen_aux), dtype_code(xc), stream()),
+          "ptj_dropout_add_layernorm")
+    return y, h, keep
+
+
 def _layernorm_bwd(dloss_dx, layer_params, x, want_dx, want_p, residual=None, drop=None, drop_sum=False):
     require_gpu(dloss_dx, x)
     d2, x2 = _rows2d(dloss_dx), _rows2d(x)
@@ -470,8 +494,13 @@ def embed_bkwd_add_t(dwemb, d, y):
     return dwemb
 
 
-def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
-    """One block (model_triton.py:2214-2223).  y [B,T,D] -> (y_out, acts)."""
+def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None, h1=None, next_ln=None):
+    """One block (model_triton.py:2214-2223).  y [B,T,D] -> (y_out, acts).
+
+    `h1`, if given, is t_layernorm_fwd_t((ln1g, ln1b), y) already computed by the producer
+    of y; `next_ln` = (gamma, beta) of the LayerNorm that consumes y_out asks for the same
+    service: the result is then (y_out, acts, layernorm(y_out)), the norm coming out of the
+    pass that forms y_out."""
     if not train:
         p_gen_aux = [0, 0, 0]
     ln1g, ln1b, wqkv, wo, ln2g, ln2b, w1, b1, w2, b2 = layer_params
@@ -479,7 +508,10 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
     H, _, dh, _ = wqkv.shape
     N = B * T
     x_in = y.reshape(N, D)
-    h1 = t_layernorm_fwd_t((ln1g, ln1b), x_in)
+    if h1 is None:
+        h1 = t_layernorm_fwd_t((ln1g, ln1b), x_in)
+    else:
+        h1 = h1.reshape(N, D)
     qkv = matmul_t(h1, wqkv.view(H * 3 * dh, D).t())                     # [N, H*3*dh]
     v5 = qkv.view(B, T, H, 3, dh)
     q, k, v = (v5[:, :, :, c].permute(0, 2, 1, 3) for c in range(3))     # [B,H,T,dh] views
@@ -487,13 +519,17 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None):
     o4 = o2.view(B, T, H, dh).permute(0, 2, 1, 3)
     _, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux[0], out=o4)
     a_out = matmul_t(o2, wo.t())
-    x_mid, keep1 = dropout_add_t(a_out, x_in, train, p_gen_aux[1], want_keep=True)
-    h2 = t_layernorm_fwd_t((ln2g, ln2b), x_mid)
+    x_mid, h2, keep1 = dropout_add_layernorm_t(a_out, x_in, (ln2g, ln2b), train, p_gen_aux[1], want_keep=True)
     f1 = torch.empty((N, w1.shape[0]), dtype=y.dtype, device=y.device)
     g1 = matmul_t(h2, w1.t(), b1, gelu=True, pre_out=f1)               # bias + GELU epilogue, both kept
     f2 = matmul_t(g1, w2.t(), b2)
-    x_out, keep2 = dropout_add_t(f2, x_mid, train, p_gen_aux[2], want_keep=True)
+    if next_ln is not None:
+        x_out, h_next, keep2 = dropout_add_layernorm_t(f2, x_mid, next_ln, train, p_gen_aux[2], want_keep=True)
+    else:
+        x_out, keep2 = dropout_add_t(f2, x_mid, train, p_gen_aux[2], want_keep=True)
     acts = (x_in, h1, qkv, o2, ms, ls, x_mid, h2, f1, g1, keep1, keep2)
+    if next_ln is not None:
+        return x_out.view(B, T, D), acts, h_next.view(B, T, D)
     return x_out.view(B, T, D), acts
 
 
@@ -563,10 +599,16 @@ def t_gpt2_tlayers_fwd3_t(params, y, mask, indices, train=True, p_gen_aux=None):
     assert T <= params[1][0].shape[0], "sequence longer than the positional table"
     x = embed_pos_dropout_t(params[0][0], params[1][0], y, train, p_gen_aux[0])
     layer_acts = []
-    for i, lp in enumerate(params[2:-1]):
-        x, a = t_gpt2_tlayer_fwd3_t(lp, x, mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i])
+    layers = params[2:-1]
+    h = None                                   # layernorm of x by the LayerNorm that reads it next
+    for i, lp in enumerate(layers):
+        # the pass that forms a block's output also applies the next norm (the next block's
+        # first one, or the final one)
+        nxt = (layers[i + 1][0], layers[i + 1][1]) if i + 1 < len(layers) else params[-1]
+        x, a, h = t_gpt2_tlayer_fwd3_t(lp, x, mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i], h1=h, next_ln=nxt)
         layer_acts.append(a)
-    h = t_layernorm_fwd_t(params[-1], x)
+    if h is None:
+        h = t_layernorm_fwd_t(params[-1], x)
     return h, [layer_acts, x]
 
 

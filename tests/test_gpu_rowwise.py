@@ -70,6 +70,26 @@ def test_gelu(mt, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4096, 768), (333, 768), (64, 1024), (17, 4096), (5, 100), (3, 1001), (2, 16384)])
+def test_dropout_add_layernorm_matches_separate_calls(mt, dtype, shape):
+    """Residual update + LayerNorm in one pass: bit-exact against dropout_add_t followed by
+    t_layernorm_fwd_t (both outputs and the recorded keep bytes), train and eval."""
+    g = gen(31)
+    x, res = randn(g, *shape, dtype=dtype).to(DEV), randn(g, *shape, dtype=dtype).to(DEV)
+    gamma, beta = randn(g, shape[1], dtype=dtype).to(DEV), randn(g, shape[1], dtype=dtype).to(DEV)
+    for train in (True, False):
+        y0, keep0 = mt.dropout_add_t(x, res, train, 9191, want_keep=True)
+        h0 = mt.t_layernorm_fwd_t((gamma, beta), y0)
+        y1, h1, keep1 = mt.dropout_add_layernorm_t(x, res, (gamma, beta), train, 9191, want_keep=True)
+        assert torch.equal(y0, y1) and torch.equal(h0, h1)
+        assert (keep0 is None) == (keep1 is None)
+        if keep0 is not None:
+            assert torch.equal(keep0, keep1)
+        y2, h2, keep2 = mt.dropout_add_layernorm_t(x, res, (gamma, beta), train, 9191)
+        assert keep2 is None and torch.equal(y0, y2) and torch.equal(h0, h2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(16384, 3072), (1000, 768), (37, 101), (1, 8), (2, 3, 64)])
 def test_gelu_bwd_with_colsum_matches_separate_calls(mt, dtype, shape):
     """The fused entry point writes exactly the dx of t_gelu_bkwd2_t and the column sums of
