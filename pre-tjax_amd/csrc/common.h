@@ -153,7 +153,7 @@ __device__ __forceinline__ bool philox_keep(uint32_t offset, uint32_t k0, uint32
 struct SigPair { float s, om; };  // s = sigmoid(2z), om = 1 - s
 __device__ __forceinline__ SigPair sigmoid2z(float z) {
     const float a = __expf(-2.0f * fabsf(z));
-    const float r = 1.0f / (1.0f + a);
+    const float r = __builtin_amdgcn_rcpf(1.0f + a);   // denominator in [1, 2]: the 1-ulp hardware reciprocal
     SigPair o;
     o.s = z >= 0.f ? r : a * r;
     o.om = z >= 0.f ? a * r : r;

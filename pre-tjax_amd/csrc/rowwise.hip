@@ -633,53 +633,106 @@ __global__ __launch_bounds__(RED_THREADS) void colsum_stage2_kernel(const float*
 }
 
 // GELU backward with the column sums of its own output (the bias gradient of the linear
-// layer in front of the GELU) in the colsum_stage1 geometry: block (bx, by) handles rows
-// [by*rps, (by+1)*rps) of its 128*VEC columns, writes dx and leaves the sums of the stored
-// (storage-rounded) dx values in part[by][col].
-template <typename T, int VEC>
-__global__ __launch_bounds__(128) void gelu_bwd_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                                              T* __restrict__ dx, float* __restrict__ part,
-                                                              int64_t rows, int cols, int rows_per_split) {
-    const int c0 = (blockIdx.x * 128 + threadIdx.x) * VEC;
-    if (c0 >= cols) return;
-    const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+// layer in front of the GELU).  A workgroup owns whole rows: `tpr` threads cover a row
+// (thread t the 16-byte vectors t, t + tpr, ... : contiguous accesses) and the workgroup
+// holds blockDim / tpr such row slots, which take the rows of the workgroup's range
+// [b*rps, (b+1)*rps) in turn.  dx is written, the sums of the stored (storage-rounded) dx
+// values are folded over the slots through LDS in slot order and left in part[b][col].
+// NV = vectors per thread.
+constexpr int GELU_CS_MAX_LDS_COLS = 8192;   // floats of LDS for the slot fold
+template <typename T, int VEC, int NV>
+__global__ __launch_bounds__(1024) void gelu_bwd_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                               T* __restrict__ dx, float* __restrict__ part,
+                                                               int64_t rows, int cols, int rows_per_split, int tpr) {
+    __shared__ float red[GELU_CS_MAX_LDS_COLS];
+    const int nvec = cols / VEC;
+    const int slots = blockDim.x / tpr, slot = threadIdx.x / tpr, tx = threadIdx.x - slot * tpr;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_split;
     const int64_t r1 = r0 + rows_per_split < rows ? r0 + rows_per_split : rows;
-    float acc[VEC];
+    float acc[NV][VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    constexpr int U = 4;   // independent rows in flight per thread
-    int64_t r = r0;
-    for (; r + U <= r1; r += U) {
-        float v[U][VEC], d[U][VEC];
+    for (int k = 0; k < NV; ++k)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            load_vec<T, VEC>(x + (r + u) * (int64_t)cols + c0, v[u]);
-            load_vec<T, VEC>(dy + (r + u) * (int64_t)cols + c0, d[u]);
-        }
+        for (int j = 0; j < VEC; ++j) acc[k][j] = 0.f;
+    constexpr int U = NV == 1 ? 4 : 2;   // independent rows in flight per thread
+    int64_t r = r0 + slot;
+    for (; r + (int64_t)(U - 1) * slots < r1; r += (int64_t)U * slots) {
+        float v[U][NV][VEC], d[U][NV][VEC];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int vi = tx + k * tpr;
+                const int vc = vi < nvec ? vi : nvec - 1;
+                load_vec<T, VEC>(x + (r + u * slots) * (int64_t)cols + (int64_t)vc * VEC, v[u][k]);
+                load_vec<T, VEC>(dy + (r + u * slots) * (int64_t)cols + (int64_t)vc * VEC, d[u][k]);
+            }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int vi = tx + k * tpr;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    d[u][k][j] = to_f32(from_f32<T>(d[u][k][j] * gelu_grad_f(v[u][k][j])));
+                    acc[k][j] += d[u][k][j];
+                }
+                if (vi < nvec) store_vec<T, VEC>(dx + (r + u * slots) * (int64_t)cols + (int64_t)vi * VEC, d[u][k]);
+            }
+    }
+    for (; r < r1; r += slots) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int vi = tx + k * tpr;
+            const int vc = vi < nvec ? vi : nvec - 1;
+            float v[VEC], d[VEC];
+            load_vec<T, VEC>(x + r * (int64_t)cols + (int64_t)vc * VEC, v);
+            load_vec<T, VEC>(dy + r * (int64_t)cols + (int64_t)vc * VEC, d);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                d[u][j] = to_f32(from_f32<T>(d[u][j] * gelu_grad_f(v[u][j])));
-                acc[j] += d[u][j];
+                d[j] = to_f32(from_f32<T>(d[j] * gelu_grad_f(v[j])));
+                acc[k][j] += d[j];
             }
-            store_vec<T, VEC>(dx + (r + u) * (int64_t)cols + c0, d[u]);
+            if (vi < nvec) store_vec<T, VEC>(dx + r * (int64_t)cols + (int64_t)vi * VEC, d);
         }
     }
-    for (; r < r1; ++r) {
-        float v[VEC], d[VEC];
-        load_vec<T, VEC>(x + r * (int64_t)cols + c0, v);
-        load_vec<T, VEC>(dy + r * (int64_t)cols + c0, d);
+    // fold the slots in slot order (only used with slots > 1, which the host allows when
+    // the row fits the LDS array)
+    for (int s = 1; s < slots; ++s) {
+        if (slot == s) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-            d[j] = to_f32(from_f32<T>(d[j] * gelu_grad_f(v[j])));
-            acc[j] += d[j];
+            for (int k = 0; k < NV; ++k) {
+                const int vi = tx + k * tpr;
+                if (vi < nvec) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) red[vi * VEC + j] = acc[k][j];
+                }
+            }
         }
-        store_vec<T, VEC>(dx + r * (int64_t)cols + c0, d);
-    }
-    float* dst = part + (int64_t)blockIdx.y * cols + c0;
+        __syncthreads();
+        if (slot == 0) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) dst[j] = acc[j];
+            for (int k = 0; k < NV; ++k) {
+                const int vi = tx + k * tpr;
+                if (vi < nvec) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[k][j] += red[vi * VEC + j];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (slot == 0) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int vi = tx + k * tpr;
+            if (vi < nvec) {
+                float* dst = part + (int64_t)blockIdx.x * cols + (int64_t)vi * VEC;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) dst[j] = acc[k][j];
+            }
+        }
+    }
 }
 
 inline void colsum_geometry(int64_t rows, int64_t cols, int vec, int* gx, int* splits, int* rps) {
@@ -717,22 +770,57 @@ int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t row
 }
 
 template <typename T>
+int gelu_impl(const void* dy, const void* x, void* out, int64_t n, bool bwd, hipStream_t st);
+
+// Rows per workgroup of the fused GELU backward: two workgroups per CU, at most 512 partial
+// rows.
+inline void gelu_bwd_colsum_geometry(int64_t rows, int64_t max_splits, int* splits, int* rps) {
+    int64_t s = (rows + 31) / 32;
+    if (s > 512) s = 512;
+    if (s > max_splits) s = max_splits;   // the partials must fit the caller's workspace
+    if (s < 1) s = 1;
+    *rps = (int)((rows + s - 1) / s);
+    *splits = (int)((rows + *rps - 1) / *rps);
+}
+
+template <typename T>
 int gelu_bwd_colsum_impl(const void* dy, const void* x, void* dx, void* colsum, void* ws, size_t ws_bytes, int64_t rows,
                          int64_t cols, hipStream_t st) {
     constexpr int FV = VecOf<T>::N;
     const bool vok = (cols % FV == 0) && ptj_aligned16(x) && ptj_aligned16(dy) && ptj_aligned16(dx);
-    const int vec = vok ? FV : 1;
-    int gx, splits, rps;
-    colsum_geometry(rows, cols, vec, &gx, &splits, &rps);
-    const size_t need = (size_t)splits * cols * sizeof(float);
-    if (!ws || ws_bytes < need)
-        return ptj_set_error(PTJ_ERR_WORKSPACE, "gelu_bwd_colsum: workspace %zu < %zu bytes", ws_bytes, need);
-    if (vok)
-        hipLaunchKernelGGL((gelu_bwd_colsum_kernel<T, FV>), dim3(gx, splits), dim3(128), 0, st, (const T*)dy, (const T*)x,
-                           (T*)dx, (float*)ws, rows, (int)cols, rps);
-    else
-        hipLaunchKernelGGL((gelu_bwd_colsum_kernel<T, 1>), dim3(gx, splits), dim3(128), 0, st, (const T*)dy, (const T*)x,
-                           (T*)dx, (float*)ws, rows, (int)cols, rps);
+    int splits, rps;
+    if (!ws || ws_bytes < (size_t)cols * sizeof(float))
+        return ptj_set_error(PTJ_ERR_WORKSPACE, "gelu_bwd_colsum: workspace %zu < %zu bytes", ws_bytes,
+                             (size_t)cols * sizeof(float));
+    gelu_bwd_colsum_geometry(rows, (int64_t)(ws_bytes / ((size_t)cols * sizeof(float))), &splits, &rps);
+    const int64_t nvec = vok ? cols / FV : cols;
+    // threads per row: a multiple of 64 that covers the row in one, two or four sweeps
+    const int nv = nvec <= 512 ? 1 : nvec <= 1024 ? 2 : 4;
+    const int tpr = (int)(((nvec + nv - 1) / nv + 63) / 64 * 64);
+    if (tpr > 512) {
+        // wider rows: separate passes
+        int rc = gelu_impl<T>(dy, x, dx, rows * cols, true, st);
+        if (rc != PTJ_OK) return rc;
+        return colsum_impl<T>(dx, colsum, ws, ws_bytes, rows, cols, cols, st);
+    }
+    // row slots per workgroup: up to 1024 threads, as long as a row fits the fold buffer
+    int slots = 1024 / tpr;
+    if (slots > 4) slots = 4;
+    if (cols > GELU_CS_MAX_LDS_COLS || slots < 1) slots = 1;
+    const int threads = tpr * slots;
+#define LAUNCH(V_, NV_)                                                                                          \
+    hipLaunchKernelGGL((gelu_bwd_colsum_kernel<T, V_, NV_>), dim3(splits), dim3(threads), 0, st, (const T*)dy,   \
+                       (const T*)x, (T*)dx, (float*)ws, rows, (int)cols, rps, tpr)
+    if (vok) {
+        if (nv == 1) LAUNCH(FV, 1);
+        else if (nv == 2) LAUNCH(FV, 2);
+        else LAUNCH(FV, 4);
+    } else {
+        if (nv == 1) LAUNCH(1, 1);
+        else if (nv == 2) LAUNCH(1, 2);
+        else LAUNCH(1, 4);
+    }
+#undef LAUNCH
     PTJ_CHECK_LAUNCH();
     hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
                        (const float*)ws, splits, (int)cols, (T*)colsum);
