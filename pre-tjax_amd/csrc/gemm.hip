@@ -544,9 +544,32 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
     const int total = num_m * num_n;
     const int work = total * g.splits;
     for (int item = blockIdx.x; item < work; item += gridDim.x) {
-        const int z = item / total;
-        int row0, col0;
-        tile_origin(item - z * total, total, num_m, num_n, row0, col0);
+        int z = 0, row0, col0;
+        if (g.splits > 1) {
+            // K-split products are bound by operand traffic: the items of one XCD (a contiguous
+            // index range after the regrouping, all resident at once) are chosen to share operand
+            // slices.  Index order: the tiles along the smaller C dimension fastest (they share
+            // the K slice of the larger operand), then the tiles along the larger one, then the
+            // K split -- so every slice of the larger operand is fetched by one XCD only.
+            const int chunk = work >> 3, rem = work & 7, x = item & 7;
+            const int idx = x * chunk + (x < rem ? x : rem) + (item >> 3);
+            int tile_m, tile_n;
+            if (g.n >= g.m) {
+                tile_n = idx % num_n;
+                const int pair = idx / num_n;
+                tile_m = pair % num_m;
+                z = pair / num_m;
+            } else {
+                tile_m = idx % num_m;
+                const int pair = idx / num_m;
+                tile_n = pair % num_n;
+                z = pair / num_n;
+            }
+            row0 = tile_m * BM;
+            col0 = tile_n * BN;
+        } else {
+            tile_origin(item, total, num_m, num_n, row0, col0);
+        }
 
         const int kbeg = z * g.k_per_split;
         const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
