@@ -62,6 +62,9 @@ struct GemmArgs {
     int64_t c_rs;
     int k_per_split;      // multiple of BK
     int splits;
+    int tail_first;       // > 0: tiles [tail_first, tiles) -- the last, partly filled round -- are K-split
+    int tail_splits;      //      into tail_splits items each (dense fp32 partial tiles in `partial`)
+    int tail_kps;         //      of tail_kps contraction elements (multiple of BK)
     int stream;           // no K split and K is a whole even number of panels: tiles are pipelined back to back
     int vec_out;          // every output (C, pre-activation, partials) and the bias allow aligned 16-byte rows
     int epilogue;
@@ -386,11 +389,11 @@ __device__ __forceinline__ void tile_origin(int pid, int total, int num_m, int n
 // Bias / GELU are applied in registers, the block is converted to the output type,
 // staged in the wave-private LDS area and written back as 16-byte vectors that run
 // along whole 96-column rows.  Only wave-local ordering is needed.
-template <typename T, bool BIAS>
+template <typename T, bool BIAS, bool SPLIT = true>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
                                               int row0, int col0, int z) {
     const bool full = row0 + BM <= g.n && col0 + BN <= g.m && g.vec_out;
-    if (g.partial != nullptr) {
+    if (SPLIT && g.partial != nullptr) {
         float* part = g.partial + (int64_t)z * g.n * (int64_t)g.m;
         if (full) gemm_store_block<float, T, false, false, true>(g, acc, smem, row0, col0, part, g.m);
         else gemm_store_block<float, T, false, false, false>(g, acc, smem, row0, col0, part, g.m);
@@ -509,7 +512,7 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
 #undef ROW_B
         }
         load_bias_quads<T, CLAMP>(g, ncol0, braw);
-        gemm_epilogue<T, false>(g, acc, smem, row0, col0, 0);
+        gemm_epilogue<T, false, false>(g, acc, smem, row0, col0, 0);
         if (!more) break;
         item = nitem;
         row0 = nrow0;
@@ -542,10 +545,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
 
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     const int total = num_m * num_n;
-    const int work = total * g.splits;
+    const int work = g.tail_splits > 1 ? g.tail_first + (total - g.tail_first) * g.tail_splits : total * g.splits;
     for (int item = blockIdx.x; item < work; item += gridDim.x) {
         int z = 0, row0, col0;
-        if (g.splits > 1) {
+        int kbeg = 0, kend = g.k;
+        float* tail_part = nullptr;
+        if (g.tail_splits > 1 && item >= g.tail_first) {
+            // a tile of the last round: one of its K slices, written as a dense partial tile
+            const int r = item - g.tail_first;
+            const int t = r / g.tail_splits;
+            z = r - t * g.tail_splits;
+            tile_origin(g.tail_first + t, total, num_m, num_n, row0, col0);
+            kbeg = z * g.tail_kps;
+            kend = (kbeg + g.tail_kps) < g.k ? (kbeg + g.tail_kps) : g.k;
+            tail_part = g.partial + (int64_t)r * (BM * BN);
+        } else if (g.splits > 1) {
             // K-split products are bound by operand traffic: the items of one XCD (a contiguous
             // index range after the regrouping, all resident at once) are chosen to share operand
             // slices.  Index order: the tiles along the smaller C dimension fastest (they share
@@ -567,12 +581,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
             }
             row0 = tile_m * BM;
             col0 = tile_n * BN;
+            kbeg = z * g.k_per_split;
+            kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
         } else {
             tile_origin(item, total, num_m, num_n, row0, col0);
         }
-
-        const int kbeg = z * g.k_per_split;
-        const int kend = (kbeg + g.k_per_split) < g.k ? (kbeg + g.k_per_split) : g.k;
         const int nk = (kend - kbeg + BK - 1) / BK;
 
         f32x16 acc[TN][TM];
@@ -596,7 +609,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
         } else {
             gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
         }
-        gemm_epilogue<T, true>(g, acc, smem, row0, col0, z);
+        if (tail_part != nullptr) gemm_store_block<float, T, false, false, true>(g, acc, smem, 0, 0, tail_part, BN);
+        else if (g.tail_splits > 1) gemm_epilogue<T, true, false>(g, acc, smem, row0, col0, z);
+        else gemm_epilogue<T, true, true>(g, acc, smem, row0, col0, z);
     }
 }
 
@@ -618,6 +633,28 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     }
 }
 
+// Second stage for the K-split tiles of the last round: tile t (work item tail_first + t) =
+// epilogue(sum_z partial[t*splits + z]) in z order; partial tiles are dense BM x BN.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const GemmArgs g) {
+    const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
+    const int t = blockIdx.x;
+    int row0, col0;
+    tile_origin(g.tail_first + t, num_m * num_n, num_m, num_n, row0, col0);
+    const float* base = g.partial + (int64_t)t * g.tail_splits * (BM * BN);
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < BM * BN; i += gridDim.y * 256) {
+        const int r = i / BN, c = i - r * BN;
+        const int row = row0 + r, col = col0 + c;
+        if (row >= g.n || col >= g.m) continue;
+        float s = 0.f;
+        for (int z = 0; z < g.tail_splits; ++z) s += base[(int64_t)z * (BM * BN) + i];
+        if (g.epilogue != PTJ_EPI_NONE) s += to_f32(((const T*)g.bias)[col]);
+        if (g.c_aux != nullptr) ((T*)g.c_aux)[(int64_t)row * g.c_aux_rs + col] = from_f32<T>(s);
+        if (g.epilogue == PTJ_EPI_BIAS_GELU) s = gelu_f(s);
+        ((T*)g.c)[(int64_t)row * g.c_rs + col] = from_f32<T>(s);
+    }
+}
+
 template <typename T>
 int pick_mode(const void* p, int64_t s_row, int64_t s_k) {
     constexpr int VEC = VecOf<T>::N;
@@ -631,7 +668,8 @@ template <typename T>
 int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     const int am = pick_mode<T>(g.a, g.a_row, g.a_k), bm = pick_mode<T>(g.b, g.b_row, g.b_k);
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
-    const int64_t work = (int64_t)num_m * num_n * splits;
+    int64_t work = (int64_t)num_m * num_n * splits;
+    if (g.tail_splits > 1) work = g.tail_first + ((int64_t)num_m * num_n - g.tail_first) * g.tail_splits;
     dim3 grid((unsigned)(work < NUM_CUS ? work : NUM_CUS)), block(GEMM_THREADS);
 #define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD>), grid, block, 0, st, g)
     switch (am * 3 + bm) {
@@ -654,6 +692,11 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
         hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st,
                            (const float*)g.partial, splits, g.n, g.m, (T*)g.c, g.c_rs, (const T*)g.bias, g.epilogue,
                            (T*)g.c_aux, g.c_aux_rs);
+        PTJ_CHECK_LAUNCH();
+    }
+    if (g.tail_splits > 1) {
+        hipLaunchKernelGGL((gemm_tail_reduce_kernel<T>), dim3((unsigned)(num_m * num_n - g.tail_first), 12), dim3(256), 0,
+                           st, g);
         PTJ_CHECK_LAUNCH();
     }
     return PTJ_OK;
@@ -683,6 +726,30 @@ int choose_splits(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes) {
     return best;
 }
 
+// K split of the last, partly filled round of tiles.  When the tile count is not a multiple
+// of the CU count and the contraction is long, the leftover tiles would keep a few CUs busy
+// for a whole tile time; they are cut into `*splits` K slices each so that the last round
+// fills the chip and takes 1/splits of a tile time.  Returns the workspace bytes (0 = off).
+size_t choose_tail_split(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes, int* first, int* splits, int* kps) {
+    constexpr int CUS = 256;
+    const int64_t tiles = ((n + BM - 1) / BM) * ((m + BN - 1) / BN);
+    const int bk = BKB / elt;
+    const int64_t panels = k / bk;
+    *first = 0; *splits = 1; *kps = 0;
+    const int64_t tail = tiles % CUS, rounds = tiles / CUS;
+    if (tiles <= CUS || tail == 0 || tail > CUS / 2 || rounds > 16 || panels < 32 || k % bk != 0) return 0;
+    int64_t s = CUS / tail;
+    if (s > panels / 8) s = panels / 8;
+    if (s > 32) s = 32;
+    if (s < 2) return 0;
+    const int64_t per = ((panels + s - 1) / s) * bk;
+    s = (k + per - 1) / per;
+    const size_t need = (size_t)tail * s * BM * BN * sizeof(float);
+    if (s < 2 || need > ws_bytes) return 0;
+    *first = (int)(tiles - tail); *splits = (int)s; *kps = (int)per;
+    return need;
+}
+
 }  // namespace
 
 extern "C" {
@@ -691,7 +758,9 @@ size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype) {
     if (n <= 0 || m <= 0 || k <= 0) return 0;
     const int elt = dtype == PTJ_BF16 ? 2 : 4;
     const int s = choose_splits(n, m, k, elt, (size_t)-1);
-    return s > 1 ? (size_t)s * n * m * sizeof(float) : 0;
+    if (s > 1) return (size_t)s * n * m * sizeof(float);
+    int first, ts, tkps;
+    return choose_tail_split(n, m, k, elt, (size_t)-1, &first, &ts, &tkps);
 }
 
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n, int64_t m, int64_t k, int64_t a_rs,
@@ -727,6 +796,9 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     if (kps < 1) kps = bk;  // k == 0: one empty pass writes bias / zeros
     g.k_per_split = (int)kps;
     g.splits = splits;
+    g.tail_first = 0; g.tail_splits = 1; g.tail_kps = 0;
+    if (splits == 1 && workspace && ptj_aligned16(workspace))
+        choose_tail_split(n, m, k, elt, workspace_bytes, &g.tail_first, &g.tail_splits, &g.tail_kps);
     {
         const int64_t v = 16 / elt;
         bool ok = ptj_aligned16(c) && c_rs % v == 0;
@@ -735,9 +807,9 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
         if (splits > 1) ok = ok && ptj_aligned16(workspace) && m % 4 == 0;
         g.vec_out = ok ? 1 : 0;
     }
-    g.partial = splits > 1 ? (float*)workspace : nullptr;
+    g.partial = (splits > 1 || g.tail_splits > 1) ? (float*)workspace : nullptr;
     // streamed tiles need whole, evenly many K panels (the two-step loop body) and vector-aligned outputs
-    g.stream = (splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
+    g.stream = (splits == 1 && g.tail_splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
 }

@@ -69,6 +69,23 @@ def test_gemm_split_k_dw_shapes(mt, dtype, n, m, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,m,k,layout", [(16640, 768, 2048, "tn"), (16500, 770, 2048, "nt"), (16640, 768, 4096, "nn")])
+def test_gemm_split_last_round(mt, dtype, n, m, k, layout):
+    """More tiles than CUs with a small remainder and a long contraction: the tiles of the
+    last round are K-split (dense partial tiles + a second stage), with and without tiles that
+    cross the border of C, with bias; the result does not depend on the run."""
+    g = gen(13)
+    a = randn(g, n, k, dtype=dtype, std=0.5) if layout[0] == "n" else randn(g, k, n, dtype=dtype, std=0.5).t()
+    b = randn(g, k, m, dtype=dtype, std=0.5) if layout[1] == "n" else randn(g, m, k, dtype=dtype, std=0.5).t()
+    bias = randn(g, m, dtype=dtype)
+    ad = (a.t().contiguous().to(DEV).t() if layout[0] == "t" else a.to(DEV))
+    bd = (b.t().contiguous().to(DEV).t() if layout[1] == "t" else b.to(DEV))
+    c = mt.matmul_t(ad, bd, bias.to(DEV))
+    check(c, a, b, dtype, bias=bias)
+    assert torch.equal(c, mt.matmul_t(ad, bd, bias.to(DEV)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_bias_gelu_and_ffn(mt, dtype):
     g = gen(12)
     x = randn(g, 4, 96, 768, dtype=dtype)
