@@ -409,15 +409,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&
 }
 
 // Bias of this lane's 12 column quads of the tile at column col0, in storage type (zeros
-// without a bias).  CLAMP: the tile may cross the right border; columns past it re-read
+// without a bias, or on request: K slices get their bias in the second stage).  CLAMP: the tile may cross the right border; columns past it re-read
 // the last valid one.
 template <typename T, bool CLAMP>
-__device__ __forceinline__ void load_bias_quads(const GemmArgs& g, int col0, Pack<T, 4> (&b)[TN * 4]) {
+__device__ __forceinline__ void load_bias_quads(const GemmArgs& g, int col0, Pack<T, 4> (&b)[TN * 4], bool zero) {
     const int tid = fresh_tid();
     const int lg = (tid & 63) >> 5, wn = (tid >> 6) % WAVES_N;
     const int gcol0 = col0 + wn * 96 + lg * 4;
     const T* bias = (const T*)g.bias;
-    if (g.epilogue == PTJ_EPI_NONE) {
+    if (zero || g.epilogue == PTJ_EPI_NONE) {
 #pragma unroll
         for (int q = 0; q < TN * 4; ++q)
 #pragma unroll
@@ -456,7 +456,8 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
     constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     const int total = num_m * num_n;
-    const int nk = g.k / BK;
+    // work items: whole tiles, then (with a K-split last round) the K slices of its tiles
+    const int work = g.tail_splits > 1 ? g.tail_first + (total - g.tail_first) * g.tail_splits : total;
     const T* A = (const T*)g.a;
     const T* B = (const T*)g.b;
     char* sA = smem;
@@ -464,20 +465,38 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
     TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1;
     TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1;
     typename Frag<T>::type fa[2][TM], fb[TN], fx[TN];
+    // item -> tile origin, first contraction element, number of panels (even), partial tile
+#define STREAM_ITEM(ITEM, ROW0, COL0, KBEG, NK, PART)                                                    \
+    do {                                                                                                 \
+        if (g.tail_splits > 1 && (ITEM) >= g.tail_first) {                                               \
+            const int r__ = (ITEM) - g.tail_first;                                                       \
+            const int t__ = r__ / g.tail_splits, z__ = r__ - t__ * g.tail_splits;                        \
+            tile_origin(g.tail_first + t__, total, num_m, num_n, ROW0, COL0);                            \
+            KBEG = z__ * g.tail_kps;                                                                     \
+            NK = ((KBEG + g.tail_kps < g.k ? g.tail_kps : g.k - KBEG)) / BK;                             \
+            PART = g.partial + (int64_t)r__ * (BM * BN);                                                 \
+        } else {                                                                                         \
+            tile_origin(ITEM, total, num_m, num_n, ROW0, COL0);                                          \
+            KBEG = 0;                                                                                    \
+            NK = g.k / BK;                                                                               \
+            PART = nullptr;                                                                              \
+        }                                                                                                \
+    } while (0)
     int item = blockIdx.x;
-    int row0, col0;
-    tile_origin(item, total, num_m, num_n, row0, col0);
+    int row0, col0, kbeg, nk;
+    float* part;
+    STREAM_ITEM(item, row0, col0, kbeg, nk, part);
     Pack<T, 4> braw[TN * 4];
-    load_bias_quads<T, CLAMP>(g, col0, braw);
+    load_bias_quads<T, CLAMP>(g, col0, braw, part != nullptr);
     {
         const int tid = fresh_tid();
         const int lane = tid & 63, wave = tid >> 6;
         const int lr = lane & 31, lg = lane >> 5;
         const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
-        la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, 0, tid, g.n);
-        lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, 0, tid, g.m);
-        la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, BK, tid, g.n);
-        lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, BK, tid, g.m);
+        la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, kbeg, tid, g.n);
+        lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, kbeg, tid, g.m);
+        la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, kbeg + BK, tid, g.n);
+        lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, kbeg + BK, tid, g.m);
         la0.store(sA, tid);
         lb0.store(sB, tid);
         __syncthreads();
@@ -485,9 +504,10 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
     }
     for (;;) {
         const int nitem = item + (int)gridDim.x;
-        const bool more = nitem < total;
-        int nrow0, ncol0;
-        tile_origin(more ? nitem : item, total, num_m, num_n, nrow0, ncol0);
+        const bool more = nitem < work;
+        int nrow0, ncol0, nkbeg, nnk;
+        float* npart;
+        STREAM_ITEM(more ? nitem : item, nrow0, ncol0, nkbeg, nnk, npart);
         f32x16 acc[TN][TM];
 #pragma unroll
         for (int i = 0; i < TN; ++i)
@@ -500,7 +520,7 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
             const int lane = tid & 63, wave = tid >> 6;
             const int lr = lane & 31, lg = lane >> 5;
             const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
-#define K0_OF(KT) (((KT) < nk ? (KT) : (KT) - nk) * BK)
+#define K0_OF(KT) ((KT) < nk ? kbeg + (KT) * BK : nkbeg + ((KT) - nk) * BK)
 #define ROW_A(KT) ((KT) < nk ? row0 : nrow0)
 #define ROW_B(KT) ((KT) < nk ? col0 : ncol0)
             for (int kt = 0; kt < nk; kt += 2) {
@@ -511,13 +531,18 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
 #undef ROW_A
 #undef ROW_B
         }
-        load_bias_quads<T, CLAMP>(g, ncol0, braw);
-        gemm_epilogue<T, false, false>(g, acc, smem, row0, col0, 0);
+        load_bias_quads<T, CLAMP>(g, ncol0, braw, npart != nullptr);
+        if (part != nullptr) gemm_store_block<float, T, false, false, true>(g, acc, smem, 0, 0, part, BN);
+        else gemm_epilogue<T, false, false>(g, acc, smem, row0, col0, 0);
         if (!more) break;
         item = nitem;
         row0 = nrow0;
         col0 = ncol0;
+        kbeg = nkbeg;
+        nk = nnk;
+        part = npart;
     }
+#undef STREAM_ITEM
 }
 #undef SB
 #undef RD_A
@@ -742,8 +767,11 @@ size_t choose_tail_split(int64_t n, int64_t m, int64_t k, int elt, size_t ws_byt
     if (s > panels / 8) s = panels / 8;
     if (s > 32) s = 32;
     if (s < 2) return 0;
-    const int64_t per = ((panels + s - 1) / s) * bk;
+    int64_t per_panels = (panels + s - 1) / s;
+    per_panels += per_panels & 1;                       // the streamed loop takes panels in pairs
+    const int64_t per = per_panels * bk;
     s = (k + per - 1) / per;
+    if (panels % 2 != 0 || k - (s - 1) * per < 2 * bk) return 0;
     const size_t need = (size_t)tail * s * BM * BN * sizeof(float);
     if (s < 2 || need > ws_bytes) return 0;
     *first = (int)(tiles - tail); *splits = (int)s; *kps = (int)per;
@@ -809,7 +837,7 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     }
     g.partial = (splits > 1 || g.tail_splits > 1) ? (float*)workspace : nullptr;
     // streamed tiles need whole, evenly many K panels (the two-step loop body) and vector-aligned outputs
-    g.stream = (splits == 1 && g.tail_splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
+    g.stream = (splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
 }
