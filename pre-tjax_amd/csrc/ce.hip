@@ -161,18 +161,23 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                 }
             }
         }
+        const float m_own = m;                       // maximum of this thread's elements
         m = row_reduce<CE_THREADS, true>(m, smem);
         if (pred != nullptr) {
             // argmax = lowest column whose logit equals the row maximum
             int best = 0x7fffffff;
             if constexpr (CACHED) {
+                // only a thread that holds the maximum searches for its position (typically one
+                // thread of the row; the others skip the scan)
+                if (m_own == m) {
 #pragma unroll
-                for (int it = 0; it < ITERS; ++it)
+                    for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) {
-                        const int e = (t + it * CE_THREADS) * VEC + j - mis;
-                        if (v[it][j] == m && e < best) best = e;
-                    }
+                        for (int j = 0; j < VEC; ++j) {
+                            const int e = (t + it * CE_THREADS) * VEC + j - mis;
+                            if (v[it][j] == m && e < best) best = e;
+                        }
+                }
             } else {
                 for (int vi = t; vi < nvec; vi += CE_THREADS) {
                     float w[VEC];
@@ -184,18 +189,10 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                     }
                 }
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const int other = __shfl_xor(best, o, 64);
-                best = other < best ? other : best;
-            }
+            best = wave_min_int(best);
+            // per-wave results; folded by thread 0 after the barriers of the sum reduction below
+            // (the next write happens behind the next row's max reduction, which synchronises too)
             if ((t & 63) == 0) smin[t >> 6] = best;
-            __syncthreads();
-            if (t == 0) {
-                int b = smin[0];
-                for (int i = 1; i < CE_THREADS / 64; ++i) b = smin[i] < b ? smin[i] : b;
-                pred[row] = b;
-            }
         }
         float s = 0.f;
         if constexpr (CACHED) {
@@ -219,6 +216,11 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
         }
         s = row_reduce<CE_THREADS, false>(s, smem);  // contains __syncthreads: s_xy is visible after it
         const bool live = label != 0;
+        if (t == 0 && pred != nullptr) {
+            int b = smin[0];
+            for (int i = 1; i < CE_THREADS / 64; ++i) b = smin[i] < b ? smin[i] : b;
+            pred[row] = b;
+        }
         if (t == 0) row_loss[row] = live ? -(s_xy - m - logf(s)) : 0.f;
         const float scale = live ? inv_cnt / s : 0.f;
 

@@ -90,6 +90,16 @@ __device__ __forceinline__ float wave_max(float v) {
     return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
+__device__ __forceinline__ int wave_min_int(int v) {
+    auto mv = [](int x, int y) { return y < x ? y : x; };
+    v = mv(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));
+    v = mv(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));
+    v = mv(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false));
+    v = mv(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false));
+    return mv(mv(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+              mv(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
 // Reduction over the TPR threads that share one row.  TPR == 64: one wave, no LDS.
 // TPR > 64: TPR == blockDim.x, `smem` holds TPR/64 floats per call site; every
 // thread of the block must call it (uses __syncthreads).
