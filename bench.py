@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 # Measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this benchmark (commands, per-kernel table
 # and the copy-kernel scale factors: profiles/hbm_traffic__gpt2_b16_t1024_bf16_step.md): 228.3e6 read +
 # 69.3e6 written per GEMM launch, averaged over the forward, dX and dW products of a step.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 298.8e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 237.6e6
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
@@ -74,8 +74,9 @@ def main():
                     help="only the timed training steps (for profiling): no per-kernel legs, no CPU leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (the path shards by batch; see DESIGN.md); "
-              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU (the path shards by batch: data parallel over more GPUs "
+              "needs one gradient exchange per optimizer step, which is not built); --gpus %d is not supported"
+              % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
