@@ -169,9 +169,13 @@ __device__ __forceinline__ SigPair sigmoid2z(float z) {
     o.om = z >= 0.f ? a * r : r;
     return o;
 }
+// Forward only needs s = 1 / (1 + exp(-2z)), which is accurate for every z as it stands
+// (exp overflowing to +inf gives s = 0); -2 z log2(e) = x (c1 + c3 x^2) feeds the hardware exp2.
 __device__ __forceinline__ float gelu_f(float x) {
-    constexpr float k = 0.7978845608028654f;
-    return x * sigmoid2z(k * (x + 0.044715f * x * x * x)).s;
+    constexpr float k = 0.7978845608028654f, l2e = 1.4426950408889634f;
+    constexpr float c1 = -2.0f * l2e * k, c3 = -2.0f * l2e * k * 0.044715f;
+    const float e = __builtin_amdgcn_exp2f(x * fmaf(x * x, c3, c1));
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float gelu_grad_f(float x) {
     constexpr float k = 0.7978845608028654f;

@@ -347,20 +347,23 @@ _mask_cache = {}
 def _mask_arg(mask, B, T):
     """None when `mask` is exactly the causal (lower-triangular) mask -- the kernel then
     masks by index -- else a contiguous uint8 [B,T,T] tensor.  The comparison reads the
-    mask once per distinct tensor (one host sync) and is cached on (storage, version)."""
+    mask once per distinct tensor (one host sync) and is cached on (address, version, layout).
+    A cache entry keeps its mask tensor alive: the address of a cached mask can therefore
+    not be handed to another tensor while the entry exists (a freed mask's address showing
+    up again under a different mask would otherwise be taken for the old one)."""
     if mask is None:
         return None
     assert mask.shape[-2:] == (T, T), mask.shape
-    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.device)
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
     hit = _mask_cache.get(key)
     if hit is None:
         m = mask.expand(B, T, T) if mask.dim() == 3 else mask.reshape(1, T, T).expand(B, T, T)
         tril = torch.ones(T, T, dtype=torch.bool, device=mask.device).tril_()
         if bool((m.to(torch.bool) == tril).all()):
-            hit = ("causal", None)
+            hit = ("causal", None, mask)
         else:
-            hit = ("mask", m.to(torch.bool).contiguous().view(torch.uint8))
-        if len(_mask_cache) > 64:
+            hit = ("mask", m.to(torch.bool).contiguous().view(torch.uint8), mask)
+        if len(_mask_cache) >= 8:
             _mask_cache.clear()
         _mask_cache[key] = hit
     return hit[1]

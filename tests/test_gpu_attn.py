@@ -91,6 +91,25 @@ def test_attn_padding_mask(mt, dtype, train):
     close(dv, wv, dtype, "dv")
 
 
+def test_attn_mask_detection_survives_address_reuse(mt):
+    """A causal mask is recognised once per tensor and cached; a different mask that later
+    lives at the address of a freed causal mask must not be taken for it."""
+    B, H, T = 2, 2, 256
+    qkv, _, tril = make(B, H, T, torch.float32, seed=3)
+    qd = qkv.to(DEV)
+    for _ in range(4):
+        m = tril.to(DEV)
+        o_causal, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m, False, 0)
+        del m                                            # its memory may be handed out again
+        padded = tril.clone()
+        padded[:, 128:, :128] = False
+        m2 = padded.to(DEV)
+        o_pad, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m2, False, 0)
+        close(o_causal, ops.scaled_dot_prod_attn_fwd(f64(qkv), tril, False, 0), torch.float32, "O causal")
+        close(o_pad, ops.scaled_dot_prod_attn_fwd(f64(qkv), padded, False, 0), torch.float32, "O padded")
+        del m2
+
+
 def test_attn_dropout_mask_bits(mt):
     # P with q = 0, k = 0 is uniform over visible keys; with v = one-hot(key % 64) the train-mode
     # output row i, column c is (#kept keys j<=i with j%64==c)/(i+1): recovers the keep mask exactly.
