@@ -226,9 +226,10 @@ int ptj_adamw_multi(int64_t count, float* const* p, float* const* m, float* cons
 /* Causal flash-attention forward.  q/k/v/o are [B, H, T, dh] views with explicit
  * (batch, head, row) strides and unit stride along dh -- e.g. slices of the
  * [B*T, H*3*dh] output of one fused QKV product; `mask` is NULL (pure causal:
- * key j visible to query i iff j <= i) or uint8 [B, T, T] (contiguous) that is
- * ANDed with the causal block structure exactly as the reference kernel does
- * (tiles strictly above the diagonal are never visited; model_triton.py:659-661).
+ * key j visible to query i iff j <= i) or the [B, T, T] mask (shared by the heads, as in
+ * the reference, model_triton.py:637) in the bit-packed form that ptj_attn_pack_mask
+ * writes; it is ANDed with the causal block structure exactly as the reference kernel
+ * does (tiles strictly above the diagonal are never visited; model_triton.py:659-661).
  * Saves ms (running row max of the scaled, masked scores) and ls (sum of
  * exp(score - ms)) as fp32 [BH, T].  Dropout (train != 0) keeps probability
  * (i, j) of batch-head g iff tl.rand(seed + g, i + j) > 0.1; train == 0 scales
@@ -239,7 +240,17 @@ int ptj_adamw_multi(int64_t count, float* const* p, float* const* m, float* cons
  * training path produces them.  `workspace` is needed when train != 0 only
  * (ptj_attn_workspace_bytes(B, H, T) bytes; the dropout keep bits live there). */
 size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T);
-int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mask,
+
+/* Packs a uint8 [B, T, T] mask (nonzero = visible; contiguous) for the attention kernels:
+ * one bit per (query, key), stored twice -- as words of 32 queries per key and as words of
+ * 32 keys per query -- so that a wavefront fetches the mask of a 32x32 score tile with
+ * scalar loads and applies it with lane-mask selects.  `packed` holds
+ * ptj_attn_packed_mask_bytes(B, T) bytes (a quarter of the byte mask).  T % 32 == 0.
+ * The reference passes the bool mask itself to its kernels (model_triton.py:637, 672). */
+size_t ptj_attn_packed_mask_bytes(int64_t B, int64_t T);
+int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t T, void* stream);
+
+int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint32_t* mask,
                  void* o, float* ms, float* ls, void* workspace, size_t workspace_bytes,
                  int64_t B, int64_t H, int64_t T, int64_t dh,
                  int64_t q_b_stride, int64_t q_h_stride, int64_t q_row_stride,
@@ -254,7 +265,7 @@ int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mas
  * ptj_attn_workspace_bytes(B, H, T) bytes.  Replaces
  * t_scaled_dot_prod_attn_bkwd3_k/_t (model_triton.py:829-1003). */
 int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o,
-                 const float* ms, const float* ls, const uint8_t* mask,
+                 const float* ms, const float* ls, const uint32_t* mask,
                  void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes,
                  int64_t B, int64_t H, int64_t T, int64_t dh,
                  int64_t do_b_stride, int64_t do_h_stride, int64_t do_row_stride,

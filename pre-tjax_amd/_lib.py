@@ -49,6 +49,8 @@ SIGNATURES = {
     "ptj_adamw_multi": (_int, [_i64, _p, _p, _p, _p, _p, _p, _p, _c.c_float, _c.c_float, _c.c_float, _c.c_float, _i64,
                                _int, _int, _p]),
     "ptj_attn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "ptj_attn_packed_mask_bytes": (_sz, [_i64, _i64]),
+    "ptj_attn_pack_mask": (_int, [_p, _p, _i64, _i64, _p]),
     "ptj_attn_fwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz] + [_i64] * 16 + [_int, _i64, _int, _p]),
     "ptj_attn_bwd": (_int, [_p] * 11 + [_p, _sz] + [_i64] * 28 + [_int, _i64, _int, _p]),
 }

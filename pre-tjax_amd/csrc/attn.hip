@@ -50,7 +50,10 @@ template <typename T> struct AT {
 struct AttnArgs {
     const void *q, *k, *v, *o, *d_o;
     void *out0, *out1;            // fwd: out0 = O.  bwd dkdv: out0 = dK, out1 = dV.  bwd dq: out0 = dQ
-    const uint8_t* mask;          // nullptr = causal by index
+    // nullptr = causal by index; else the mask bit-packed in both orientations (ptj_attn_pack_mask):
+    //   words [0, B*T/32*T):   word (b, q/32, k) holds M[b, 32*(q/32) + r, k] in bit r   (lane = query)
+    //   then the same amount:  word (b, k/32, q) holds M[b, q, 32*(k/32) + r] in bit r   (lane = key)
+    const uint32_t* mask;
     float *ms, *ls;               // [BH, T]
     const float* delta;           // [BH, T] rowsum(dO * O)  (backward)
     const uint32_t* keepbits;     // [BH, bitwords]  (train)
@@ -172,6 +175,16 @@ template <int C> __device__ __forceinline__ uint64_t keep_lane_mask(const KeepWo
 __device__ __forceinline__ float keep_select(float v, uint64_t mask) {
     return __builtin_amdgcn_inverse_ballot_w64(mask) ? v : 0.f;
 }
+// Attention-mask words -> lane mask of accumulator register i of a 32x32 sub-tile: the
+// register holds column c = (i/4)*8 + i%4 for lanes 0..31 and column c + 4 for lanes 32..63,
+// and word w[c] carries the mask bits of the 32 lanes' rows for column c.
+__device__ __forceinline__ uint64_t mask_lanes(const uint32_t (&w)[32], int i) {
+    const int c = (i >> 2) * 8 + (i & 3);
+    return (uint64_t)w[c] | ((uint64_t)w[c + 4] << 32);
+}
+__device__ __forceinline__ float mask_select(float v, float other, uint64_t mask) {
+    return __builtin_amdgcn_inverse_ballot_w64(mask) ? v : other;
+}
 // the 16 lane masks of sub-tile J
 template <int J, int I = 0>
 __device__ __forceinline__ void keep_masks(uint64_t (&m)[16], const KeepWords& w) {
@@ -216,6 +229,29 @@ __global__ __launch_bounds__(256) void attn_keepbits_kernel(uint32_t* __restrict
         uint32_t* dst = bits + (int64_t)bh * bitwords;
         if (w < bitwords) dst[w] = (uint32_t)m;
         if (w + 1 < bitwords) dst[w + 1] = (uint32_t)(m >> 32);
+    }
+}
+
+// ---- attention mask, bit-packed in both orientations ----------------------------------
+// out word (o, b, g, x), o = 0: bits r = mask[b, 32g + r, x] (a word per key x: 32 queries);
+//                        o = 1: bits r = mask[b, x, 32g + r] (a word per query x: 32 keys).
+__global__ __launch_bounds__(256) void attn_pack_mask_kernel(const uint8_t* __restrict__ mask,
+                                                              uint32_t* __restrict__ out, int B, int T) {
+    const int64_t per = (int64_t)B * (T >> 5) * T;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < 2 * per; i += (int64_t)gridDim.x * 256) {
+        const int o = i >= per;
+        const int64_t r = i - (o ? per : 0);
+        const int x = (int)(r % T);
+        const int g = (int)((r / T) % (T >> 5));
+        const int64_t b = r / ((int64_t)T * (T >> 5));
+        const uint8_t* m = mask + b * (int64_t)T * T;
+        uint32_t w = 0;
+        if (o == 0) {
+            for (int k = 0; k < 32; ++k) w |= (m[(int64_t)(32 * g + k) * T + x] != 0 ? 1u : 0u) << k;
+        } else {
+            for (int k = 0; k < 32; ++k) w |= (m[(int64_t)x * T + 32 * g + k] != 0 ? 1u : 0u) << k;
+        }
+        out[i] = w;
     }
 }
 
@@ -361,17 +397,16 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
                 for (int j = 0; j < 2; ++j) apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
             }
             if constexpr (HAS_MASK) {
+                // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads)
+                const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + key0;
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < 2; ++j) {
+                    uint32_t w[32];
 #pragma unroll
-                    for (int g4 = 0; g4 < 4; ++g4) {
-                        const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
-                        const uint32_t m4 =
-                            *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
+                    for (int t = 0; t < 32; ++t) w[t] = mw[j * 32 + t];
 #pragma unroll
-                        for (int b = 0; b < 4; ++b)
-                            s[j][g4 * 4 + b] = ((m4 >> (8 * b)) & 0xffu) ? s[j][g4 * 4 + b] : NEG_RAW;
-                    }
+                    for (int i = 0; i < 16; ++i) s[j][i] = mask_select(s[j][i], NEG_RAW, mask_lanes(w, i));
+                }
             }
             float tmax = s[0][0];
 #pragma unroll
@@ -523,14 +558,15 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                 uint32_t okbits = 0xffffu;
                 const bool diag = q0 + j * 32 < kw0 + 31;
                 if (diag) okbits = apply_causal<false>(s, key - q0 - j * 32 - lg * 4);
+                uint32_t mwords[32];
                 if constexpr (HAS_MASK) {
+                    // one word per query: the mask bits of the wave's 32 keys (wave-uniform loads)
+                    const uint32_t* mw = a.mask + (int64_t)a.B * (a.T >> 5) * a.T +
+                                         ((int64_t)bidx * (a.T >> 5) + (kw0u >> 5)) * a.T + q0 + j * 32;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int qq = q0 + j * 32 + (i >> 2) * 8 + lg * 4 + (i & 3);
-                        const bool ok = a.mask[((int64_t)bidx * a.T + qq) * a.T + krow] != 0;
-                        s[i] = ok ? s[i] : NEG_RAW;
-                        okbits &= ok ? 0xffffffffu : ~(1u << i);
-                    }
+                    for (int t = 0; t < 32; ++t) mwords[t] = mw[t];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[i] = mask_select(s[i], NEG_RAW, mask_lanes(mwords, i));
                 }
                 float pd[16], ds[16];
                 uint64_t km[16];
@@ -557,9 +593,13 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                         }
                     }
                 }
-                if (HAS_MASK || diag) {
+                if (diag) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
+                }
+                if constexpr (HAS_MASK) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ds[i] = mask_select(ds[i], 0.f, mask_lanes(mwords, i));
                 }
                 tp_x_regs_one(dv, base + 3 * X::NP * PANEL, pd, j, lr, lg, T());  // dV^T += dO^T P
                 tp_x_regs_one(dk, base + 2 * X::NP * PANEL, ds, j, lr, lg, T());  // dK^T += Q^T dS
@@ -656,30 +696,23 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
             rows_x_frags<T>(dp, base + X::NP * PANEL, dof, lr, lg);      // dP^T [key][query]
 
             uint32_t okbits[2] = {0xffffu, 0xffffu};
-            const bool masked = HAS_MASK || (key0 + 63 > qw0);
-            if (key0 + 63 > qw0) {
+            const bool masked = key0 + 63 > qw0;
+            if (masked) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) okbits[j] = apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
-            }
-            if constexpr (HAS_MASK) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-#pragma unroll
-                    for (int g4 = 0; g4 < 4; ++g4) {
-                        const int kb = key0 + j * 32 + g4 * 8 + lg * 4;
-                        const uint32_t m4 =
-                            *reinterpret_cast<const uint32_t*>(a.mask + ((int64_t)bidx * a.T + qrow) * a.T + kb);
-#pragma unroll
-                        for (int b = 0; b < 4; ++b) {
-                            const bool ok = ((m4 >> (8 * b)) & 0xffu) != 0;
-                            s[j][g4 * 4 + b] = ok ? s[j][g4 * 4 + b] : NEG_RAW;
-                            okbits[j] &= ok ? 0xffffffffu : ~(1u << (g4 * 4 + b));
-                        }
-                    }
             }
             float ds[2][16];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
+                uint32_t mwords[32];
+                if constexpr (HAS_MASK) {
+                    // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads)
+                    const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + key0 + j * 32;
+#pragma unroll
+                    for (int t = 0; t < 32; ++t) mwords[t] = mw[t];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[j][i] = mask_select(s[j][i], NEG_RAW, mask_lanes(mwords, i));
+                }
                 uint64_t km[16];
                 if constexpr (TRAIN) {
                     if (j == 0) keep_masks<0>(km, kw);
@@ -696,6 +729,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                 if (masked) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
+                }
+                if constexpr (HAS_MASK) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ds[j][i] = mask_select(ds[j][i], 0.f, mask_lanes(mwords, i));
                 }
             }
             tp_x_regs(dq, base + 2 * X::NP * PANEL, ds, lr, lg, T());    // dQ^T += K^T dS^T
@@ -756,7 +793,24 @@ size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T) {
     return bits_bytes(B * H, T) + delta_bytes(B * H, T);
 }
 
-int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mask, void* o, float* ms, float* ls,
+size_t ptj_attn_packed_mask_bytes(int64_t B, int64_t T) {
+    if (B < 1 || T < 32 || T % 32) return 0;
+    return (size_t)2 * B * (T / 32) * T * sizeof(uint32_t);
+}
+
+int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t T, void* stream) {
+    PTJ_CHECK_ARG(mask && packed, "attn_pack_mask: null pointer");
+    PTJ_CHECK_ARG(B >= 1 && T >= 32 && T % 32 == 0 && T < (1 << 24), "attn_pack_mask: need B >= 1 and T a multiple of 32");
+    const int64_t words = 2 * B * (T / 32) * T;
+    int64_t blocks = (words + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(attn_pack_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, mask, packed, (int)B,
+                       (int)T);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
+}
+
+int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint32_t* mask, void* o, float* ms, float* ls,
                  void* workspace, size_t workspace_bytes, int64_t B, int64_t H, int64_t T, int64_t dh,
                  int64_t q_bs, int64_t q_hs, int64_t q_rs, int64_t k_bs, int64_t k_hs, int64_t k_rs,
                  int64_t v_bs, int64_t v_hs, int64_t v_rs, int64_t o_bs, int64_t o_hs, int64_t o_rs,
@@ -790,7 +844,7 @@ int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint8_t* mas
 }
 
 int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o, const float* ms,
-                 const float* ls, const uint8_t* mask, void* dq, void* dk, void* dv, void* workspace,
+                 const float* ls, const uint32_t* mask, void* dq, void* dk, void* dv, void* workspace,
                  size_t workspace_bytes, int64_t B, int64_t H, int64_t T, int64_t dh,
                  int64_t do_bs, int64_t do_hs, int64_t do_rs, int64_t q_bs, int64_t q_hs, int64_t q_rs,
                  int64_t k_bs, int64_t k_hs, int64_t k_rs, int64_t v_bs, int64_t v_hs, int64_t v_rs,

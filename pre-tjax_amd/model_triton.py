@@ -346,7 +346,7 @@ _mask_cache = {}
 
 def _mask_arg(mask, B, T):
     """None when `mask` is exactly the causal (lower-triangular) mask -- the kernel then
-    masks by index -- else a contiguous uint8 [B,T,T] tensor.  The comparison reads the
+    masks by index -- else the mask bit-packed for the kernels (ptj_attn_pack_mask).  The comparison reads the
     mask once per distinct tensor (one host sync) and is cached on (address, version, layout).
     A cache entry keeps its mask tensor alive: the address of a cached mask can therefore
     not be handed to another tensor while the entry exists (a freed mask's address showing
@@ -354,7 +354,7 @@ def _mask_arg(mask, B, T):
     if mask is None:
         return None
     assert mask.shape[-2:] == (T, T), mask.shape
-    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device, B, T)
     hit = _mask_cache.get(key)
     if hit is None:
         m = mask.expand(B, T, T) if mask.dim() == 3 else mask.reshape(1, T, T).expand(B, T, T)
@@ -362,7 +362,11 @@ def _mask_arg(mask, B, T):
         if bool((m.to(torch.bool) == tril).all()):
             hit = ("causal", None, mask)
         else:
-            hit = ("mask", m.to(torch.bool).contiguous().view(torch.uint8), mask)
+            # bit-packed once per mask tensor, in the two orientations the kernels read
+            bytes_ = m.to(torch.bool).contiguous().view(torch.uint8)
+            packed = torch.empty(lib().ptj_attn_packed_mask_bytes(B, T) // 4, dtype=torch.int32, device=mask.device)
+            check(lib().ptj_attn_pack_mask(ptr(bytes_), ptr(packed), B, T, stream()), "ptj_attn_pack_mask")
+            hit = ("mask", packed, mask)
         if len(_mask_cache) >= 8:
             _mask_cache.clear()
         _mask_cache[key] = hit
