@@ -85,6 +85,47 @@ def test_gemm_split_last_round(mt, dtype, n, m, k, layout):
     assert torch.equal(c, mt.matmul_t(ad, bd, bias.to(DEV)))
 
 
+def _random_cases():
+    import random
+    rnd = random.Random(20240611)
+    cases = []
+    for i in range(28):
+        # many tiles (several rounds of the persistent grid at small sizes are not reachable, but
+        # streamed multi-tile workgroups, border tiles, K tails and odd panel counts all are)
+        n = rnd.choice([256, 512, 1000, 1280, 2048, 2304, 3000, 4096])
+        m = rnd.choice([192, 384, 200, 768, 770, 960, 1536])
+        k = rnd.choice([64, 128, 192, 256, 320, 768, 1000, 1024, 2048])
+        layout = rnd.choice(["nn", "nt", "tn", "tt"])
+        epi = rnd.choice(["none", "bias", "gelu", "gelu_pre"])
+        cases.append((n, m, k, layout, epi))
+    # more tiles than workgroups: every workgroup streams through two or three tiles
+    cases += [(16384, 1536, 256, "nt", "gelu_pre"), (16384, 2304, 128, "nn", "bias"), (12288, 1540, 256, "nt", "gelu"),
+              (8192, 3072, 192, "tn", "none")]
+    return cases
+
+
+@pytest.mark.parametrize("n,m,k,layout,epi", _random_cases())
+def test_gemm_random_shapes_layouts_epilogues(mt, n, m, k, layout, epi):
+    """Seeded sweep over shapes x operand layouts x epilogues in bf16 (the storage type of the
+    training step): exercises the streamed tile loop, border tiles, K tails and every epilogue
+    variant in combinations the fixed cases above do not list."""
+    dtype = torch.bfloat16
+    g = gen(n + 3 * m + 7 * k)
+    a = randn(g, n, k, dtype=dtype, std=0.5) if layout[0] == "n" else randn(g, k, n, dtype=dtype, std=0.5).t()
+    b = randn(g, k, m, dtype=dtype, std=0.5) if layout[1] == "n" else randn(g, m, k, dtype=dtype, std=0.5).t()
+    bias = randn(g, m, dtype=dtype) if epi != "none" else None
+    ad = (a.t().contiguous().to(DEV).t() if layout[0] == "t" else a.to(DEV))
+    bd = (b.t().contiguous().to(DEV).t() if layout[1] == "t" else b.to(DEV))
+    biasd = bias.to(DEV) if bias is not None else None
+    if epi == "gelu_pre":
+        pre = torch.empty(n, m, dtype=dtype, device=DEV)
+        c = mt.matmul_t(ad, bd, biasd, gelu=True, pre_out=pre)
+        check(pre, a, b, dtype, bias=bias)
+    else:
+        c = mt.matmul_t(ad, bd, biasd, gelu=(epi == "gelu"))
+    check(c, a, b, dtype, bias=bias, gelu=epi.startswith("gelu"))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_bias_gelu_and_ffn(mt, dtype):
     g = gen(12)
