@@ -103,6 +103,19 @@ __device__ __forceinline__ void rows_x_frags(f32x16 (&s)[2], const char* __restr
     }
 }
 
+// Eight floats -> eight bf16, converted two at a time (one packed conversion per pair).
+__device__ __forceinline__ bf16x8 pack8_bf16(const float* __restrict__ p) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    u32x4_t w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const f32x2_t f = {p[2 * e], p[2 * e + 1]};
+        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    return __builtin_bit_cast(bf16x8, w);
+}
+
 // o[t] += transposed_panel_rows(t*32 + lr) x p : contraction over the 32 positions of
 // sub-tile j whose values p[i] the lane holds in accumulator order
 // (position = j*32 + 8*(i/4) + 4*lg + i%4).
@@ -110,9 +123,7 @@ __device__ __forceinline__ void tp_x_regs_one(f32x16 (&o)[2], const char* __rest
                                               int j, int lr, int lg, bf16) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        bf16x8 b;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) b[e] = (bf16)p[8 * h + e];
+        const bf16x8 b = pack8_bf16(&p[8 * h]);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int row = t * 32 + lr;
@@ -166,7 +177,18 @@ template <int C> __device__ __forceinline__ uint32_t keep_win32(const KeepWords&
     return (uint32_t)(v >> (C & 31));
 }
 template <int C> __device__ __forceinline__ uint64_t keep_lane_mask(const KeepWords& w) {
-    return (uint64_t)keep_win32<C>(w) | ((uint64_t)keep_win32<C + 4>(w) << 32);
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    const u32x2_t halves = {keep_win32<C>(w), keep_win32<C + 4>(w)};
+    return __builtin_bit_cast(uint64_t, halves);
+}
+// The same for an offset that is a constant only after loop unrolling.
+__device__ __forceinline__ uint64_t keep_lane_mask_at(const KeepWords& w, int c) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    const uint64_t lo_pair = ((uint64_t)w.d1 << 32) | w.d0, hi_pair = ((uint64_t)w.d2 << 32) | w.d1;
+    const int c4 = c + 4;
+    const u32x2_t halves = {(uint32_t)((c < 32 ? lo_pair : hi_pair) >> (c & 31)),
+                            (uint32_t)((c4 < 32 ? lo_pair : hi_pair) >> (c4 & 31))};
+    return __builtin_bit_cast(uint64_t, halves);
 }
 // v where the lane's bit of `mask` is set, else 0.  The builtin turns a wave-uniform 64-bit
 // mask into a per-lane condition, i.e. one v_cndmask with the mask in scalar registers
@@ -184,14 +206,6 @@ __device__ __forceinline__ uint64_t mask_lanes(const uint32_t (&w)[32], int i) {
 }
 __device__ __forceinline__ float mask_select(float v, float other, uint64_t mask) {
     return __builtin_amdgcn_inverse_ballot_w64(mask) ? v : other;
-}
-// the 16 lane masks of sub-tile J
-template <int J, int I = 0>
-__device__ __forceinline__ void keep_masks(uint64_t (&m)[16], const KeepWords& w) {
-    if constexpr (I < 16) {
-        m[I] = keep_lane_mask<J * 32 + (I >> 2) * 8 + (I & 3)>(w);
-        keep_masks<J, I + 1>(m, w);
-    }
 }
 // p[i] = keep ? p[i] : 0 for the 16 registers of sub-tile J
 template <int J, int I = 0>
@@ -569,11 +583,6 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                     for (int i = 0; i < 16; ++i) s[i] = mask_select(s[i], NEG_RAW, mask_lanes(mwords, i));
                 }
                 float pd[16], ds[16];
-                uint64_t km[16];
-                if constexpr (TRAIN) {
-                    if (j == 0) keep_masks<0>(km, kw);
-                    else keep_masks<1>(km, kw);
-                }
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const int qi = j * 32 + g4 * 8 + lg * 4;  // first of 4 consecutive queries (tile-relative)
@@ -585,15 +594,19 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                         const int i = g4 * 4 + b;
                         const float p = fast_exp2(fmaf(s[i], sc, -m4[b])) * l4[b];
                         if constexpr (TRAIN) {
-                            pd[i] = keep_select(p, km[i]);
-                            ds[i] = p * (keep_select(dp[i], km[i]) - d4[b]);
+                            const uint64_t km = keep_lane_mask_at(kw, j * 32 + g4 * 8 + b);
+                            pd[i] = keep_select(p, km);
+                            ds[i] = p * (keep_select(dp[i], km) - d4[b]);
                         } else {
                             pd[i] = 0.9f * p;
                             ds[i] = p * fmaf(dp[i], 0.9f, -d4[b]);
                         }
                     }
                 }
-                if (diag) {
+                // Causally hidden elements: without an explicit mask every query sees its own key,
+                // so the saved row statistics are finite and p (hence dS) is exactly 0 there;
+                // with a mask a fully masked row has p != 0 and dS is cleared explicitly.
+                if (HAS_MASK && diag) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
                 }
@@ -713,20 +726,16 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 #pragma unroll
                     for (int i = 0; i < 16; ++i) s[j][i] = mask_select(s[j][i], NEG_RAW, mask_lanes(mwords, i));
                 }
-                uint64_t km[16];
-                if constexpr (TRAIN) {
-                    if (j == 0) keep_masks<0>(km, kw);
-                    else keep_masks<1>(km, kw);
-                }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const float p = fast_exp2(fmaf(s[j][i], sc, -m2)) * linv;
                     if constexpr (TRAIN)
-                        ds[j][i] = p * (keep_select(dp[j][i], km[i]) - delta);
+                        ds[j][i] = p * (keep_select(dp[j][i], keep_lane_mask_at(kw, j * 32 + (i >> 2) * 8 + (i & 3))) - delta);
                     else
                         ds[j][i] = p * fmaf(dp[j][i], 0.9f, -delta);
                 }
-                if (masked) {
+                // as in the dK/dV pass: only a masked launch can have p != 0 on hidden elements
+                if (HAS_MASK && masked) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
                 }
