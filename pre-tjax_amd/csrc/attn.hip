@@ -501,6 +501,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lq[X::NP], ld[X::NP];
     TileLoader<T, MNMAJOR, 64, ATT_THREADS> lqt[X::NP], ldt[X::NP];
     float st_m = 0.f, st_l = 1.f, st_d = 0.f;
+    // 2-byte storage without an explicit mask: 1/l goes into the exponent (p = 2^(s - m - log2 l)),
+    // one multiplication less per element.  Not with a mask: a fully masked row has m = -1e9,
+    // which would absorb log2 l.
+    constexpr bool FOLD_L = sizeof(T) == 2 && !HAS_MASK;
     const int64_t stat0 = (int64_t)bh * a.T + (tid & 63);
 #define KV_FETCH(QT)                                                                   \
     {                                                                                  \
@@ -525,7 +529,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
             ldt[p].store(base__ + (3 * X::NP + p) * PANEL, tid);                       \
         }                                                                              \
         if (tid < 64) {                                                                \
-            sstat[ST][0][tid] = st_m * LOG2E;                                          \
+            sstat[ST][0][tid] = FOLD_L ? fmaf(st_m, LOG2E, __builtin_amdgcn_logf(st_l)) : st_m * LOG2E; \
             sstat[ST][1][tid] = 1.0f / st_l;                                           \
             sstat[ST][2][tid] = st_d;                                                  \
         }                                                                              \
@@ -587,12 +591,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const int qi = j * 32 + g4 * 8 + lg * 4;  // first of 4 consecutive queries (tile-relative)
                     const f32x4 m4 = *reinterpret_cast<const f32x4*>(&sstat[st][0][qi]);
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[st][1][qi]);
+                    f32x4 l4 = {1.f, 1.f, 1.f, 1.f};
+                    if constexpr (!FOLD_L) l4 = *reinterpret_cast<const f32x4*>(&sstat[st][1][qi]);
                     const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[st][2][qi]);
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         const int i = g4 * 4 + b;
-                        const float p = fast_exp2(fmaf(s[i], sc, -m4[b])) * l4[b];
+                        float p = fast_exp2(fmaf(s[i], sc, -m4[b]));
+                        if constexpr (!FOLD_L) p *= l4[b];
                         if constexpr (TRAIN) {
                             const uint64_t km = keep_lane_mask_at(kw, j * 32 + g4 * 8 + b);
                             pd[i] = keep_select(p, km);
@@ -656,7 +662,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     load_row_frags<T>(qf, Qb + (int64_t)qrow * a.q_rs, lg);
     load_row_frags<T>(dof, dOb + (int64_t)qrow * a.do_rs, lg);
     const int64_t si = (int64_t)bh * a.T + qrow;
-    const float m2 = a.ms[si] * LOG2E, linv = 1.0f / a.ls[si], delta = a.delta[si];
+    // as in the dK/dV pass: 1/l folded into the exponent for 2-byte storage without a mask
+    constexpr bool FOLD_L = sizeof(T) == 2 && !HAS_MASK;
+    const float linv = 1.0f / a.ls[si], delta = a.delta[si];
+    const float m2 = FOLD_L ? fmaf(a.ms[si], LOG2E, __builtin_amdgcn_logf(a.ls[si])) : a.ms[si] * LOG2E;
 
     int nkt = (q0 + 128) / 64;
     if (nkt > a.T / 64) nkt = a.T / 64;
@@ -728,7 +737,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float p = fast_exp2(fmaf(s[j][i], sc, -m2)) * linv;
+                    float p = fast_exp2(fmaf(s[j][i], sc, -m2));
+                    if constexpr (!FOLD_L) p *= linv;
                     if constexpr (TRAIN)
                         ds[j][i] = p * (keep_select(dp[j][i], keep_lane_mask_at(kw, j * 32 + (i >> 2) * 8 + (i & 3))) - delta);
                     else
