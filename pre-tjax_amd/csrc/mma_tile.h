@@ -40,13 +40,8 @@ __device__ __forceinline__ void mma_chunk(f32x16& acc, const f32x4& a, const f32
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Raw bits of element e of a 16-byte vector of T, and the reverse (used by the edge and
-// transposing paths; the staging registers are plain 4 x u32 vectors so that they are
-// always promoted to registers).
-template <typename T> __device__ __forceinline__ uint32_t vec_get(const u32x4& v, int e) {
-    if constexpr (sizeof(T) == 4) return v[e];
-    else return (v[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-}
+// Sets the raw bits of element e of a 16-byte vector of T (used by the edge path; the
+// staging registers are plain 4 x u32 vectors so that they are always promoted to registers).
 template <typename T> __device__ __forceinline__ void vec_set(u32x4& v, int e, uint32_t bits) {
     if constexpr (sizeof(T) == 4) v[e] = bits;
     else v[e >> 1] = (e & 1) ? ((v[e >> 1] & 0xffffu) | (bits << 16)) : ((v[e >> 1] & 0xffff0000u) | bits);
@@ -217,8 +212,11 @@ struct TileLoader {
                             u32x4 t = {r[qi * 4 + 0][e], r[qi * 4 + 1][e], r[qi * 4 + 2][e], r[qi * 4 + 3][e]};
                             *reinterpret_cast<u32x4*>(dst) = t;
                         } else {
-                            u32x2 t = {vec_get<T>(r[qi * 4 + 0], e) | (vec_get<T>(r[qi * 4 + 1], e) << 16),
-                                       vec_get<T>(r[qi * 4 + 2], e) | (vec_get<T>(r[qi * 4 + 3], e) << 16)};
+                            // element e of two row vectors side by side: one byte permute per dword
+                            // (low halves 0x05040100, high halves 0x07060302 of {second, first})
+                            const uint32_t SEL = (e & 1) ? 0x07060302u : 0x05040100u;
+                            u32x2 t = {__builtin_amdgcn_perm(r[qi * 4 + 1][e >> 1], r[qi * 4 + 0][e >> 1], SEL),
+                                       __builtin_amdgcn_perm(r[qi * 4 + 3][e >> 1], r[qi * 4 + 2][e >> 1], SEL)};
                             *reinterpret_cast<u32x2*>(dst) = t;
                         }
                     }
