@@ -126,11 +126,9 @@ __device__ __forceinline__ void tp_x_regs_one(f32x16 (&o)[2], const char* __rest
         const bf16x8 b = pack8_bf16(&p[8 * h]);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int row = t * 32 + lr;
-            const char* rp = panels + row * BKB + lg * 8;
-            const bf16x4 lo = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h) ^ sw(row)) << 4));
-            const bf16x4 hi = *reinterpret_cast<const bf16x4*>(rp + (((4 * j + 2 * h + 1) ^ sw(row)) << 4));
-            const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            // the panel was stored with paired quads: chunk 4j + 2h + lg holds exactly the eight
+            // positions of b, in the same order
+            const bf16x8 a = read_frag<bf16>(panels, t * 32 + lr, 4 * j + 2 * h + lg);
             o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, o[t], 0, 0, 0);
         }
     }
@@ -359,7 +357,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_
     // Flat code (no closures) keeps the prefetch registers plain SSA values; the last step
     // re-fetches its own tile instead of branching.
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP];
-    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lv[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS, false, true> lv[X::NP];
 #define FWD_FETCH(KT)                                                                  \
     _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
         lk[p].load_fast(Kb, a.k_rs, 1, (KT) * 64, p * X::EPP, tid);                    \
@@ -499,7 +497,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     const int qt0 = key0 / 64, nqt = a.T / 64;
 
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lq[X::NP], ld[X::NP];
-    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lqt[X::NP], ldt[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS, false, true> lqt[X::NP], ldt[X::NP];
     float st_m = 0.f, st_l = 1.f, st_d = 0.f;
     // 2-byte storage without an explicit mask: 1/l goes into the exponent (p = 2^(s - m - log2 l)),
     // one multiplication less per element.  Not with a mask: a fully masked row has m = -1e9,
@@ -671,7 +669,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     if (nkt > a.T / 64) nkt = a.T / 64;
 
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lk[X::NP], lv[X::NP];
-    TileLoader<T, MNMAJOR, 64, ATT_THREADS> lkt[X::NP];
+    TileLoader<T, MNMAJOR, 64, ATT_THREADS, false, true> lkt[X::NP];
 #define DQ_FETCH(KT)                                                                   \
     _Pragma("unroll") for (int p = 0; p < X::NP; ++p) {                                \
         lk[p].load_fast(Kb, a.k_rs, 1, (KT) * 64, p * X::EPP, tid);                    \

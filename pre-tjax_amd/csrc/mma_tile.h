@@ -54,7 +54,12 @@ template <typename T> __device__ __forceinline__ uint32_t elem_bits(const T* p) 
 // WRAP (MNMAJOR only): when the 8x8 blocks do not divide evenly among the wavefronts, the
 // spare wavefronts repeat earlier blocks (same data to the same place) instead of idling,
 // which keeps the loader free of branches.
-template <typename T, int MODE, int ROWS, int THREADS, bool WRAP = false>
+// PAIRQ (MNMAJOR panels of 2-byte elements only): within every 16 positions of the k axis the
+// two middle quads trade places (k bits 2 and 3 swapped), so that positions {4g .. 4g+3} and
+// {8 + 4g .. 8 + 4g+3} form one 16-byte chunk -- the k order in which a lane holds a 32x32
+// accumulator tile, which lets such a tile be multiplied from registers against one
+// 16-byte LDS read per MFMA.
+template <typename T, int MODE, int ROWS, int THREADS, bool WRAP = false, bool PAIRQ = false>
 struct TileLoader {
     static constexpr int VEC = VecOf<T>::N;
     static constexpr int BK = BKB / (int)sizeof(T);
@@ -202,7 +207,9 @@ struct TileLoader {
                 const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
                 if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
                     const int prow = ((b % JB) * 8 + jc_lo) * VEC;
-                    const int kb = ((b / JB) * 8 + kq_lo) * 4 * (int)sizeof(T);  // byte offset of the quad in the row
+                    int kq = (b / JB) * 8 + kq_lo;
+                    if constexpr (PAIRQ && sizeof(T) == 2) kq = (kq & ~3) | ((kq & 1) << 1) | ((kq >> 1) & 1);
+                    const int kb = kq * 4 * (int)sizeof(T);  // byte offset of the quad in the row
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         if ((qi * VEC + e) % N != I) continue;
