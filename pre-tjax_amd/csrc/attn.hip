@@ -707,52 +707,51 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {
             const char* base = smem + st * STAGE;
-            f32x16 s[2], dp[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) s[j][e] = dp[j][e] = 0.f;
-            rows_x_frags<T>(s, base, qf, lr, lg);                        // S^T  [key][query]
-            rows_x_frags<T>(dp, base + X::NP * PANEL, dof, lr, lg);      // dP^T [key][query]
-
-            uint32_t okbits[2] = {0xffffu, 0xffffu};
-            const bool masked = key0 + 63 > qw0;
-            if (masked) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) okbits[j] = apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
-            }
-            float ds[2][16];
+            // The two 32-key halves one after the other: half the live accumulators, and a half
+            // whose keys all follow the wave's queries is skipped.
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
+                const int kh0 = key0 + j * 32;
+                if (kh0 > qw0 + 31) continue;
+                f32x16 s, dp;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
+                rows_x_frags_one<T>(s, base, qf, j, lr, lg);                       // S^T  [key][query]
+                rows_x_frags_one<T>(dp, base + X::NP * PANEL, dof, j, lr, lg);     // dP^T [key][query]
+
+                uint32_t okbits = 0xffffu;
+                const bool masked = kh0 + 31 > qw0;
+                if (masked) okbits = apply_causal<true>(s, query - kh0 - lg * 4);
                 uint32_t mwords[32];
                 if constexpr (HAS_MASK) {
                     // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads)
-                    const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + key0 + j * 32;
+                    const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + kh0;
 #pragma unroll
                     for (int t = 0; t < 32; ++t) mwords[t] = mw[t];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) s[j][i] = mask_select(s[j][i], NEG_RAW, mask_lanes(mwords, i));
+                    for (int i = 0; i < 16; ++i) s[i] = mask_select(s[i], NEG_RAW, mask_lanes(mwords, i));
                 }
+                float ds[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    float p = fast_exp2(fmaf(s[j][i], sc, -m2));
+                    float p = fast_exp2(fmaf(s[i], sc, -m2));
                     if constexpr (!FOLD_L) p *= linv;
                     if constexpr (TRAIN)
-                        ds[j][i] = p * (keep_select(dp[j][i], keep_lane_mask_at(kw, j * 32 + (i >> 2) * 8 + (i & 3))) - delta);
+                        ds[i] = p * (keep_select(dp[i], keep_lane_mask_at(kw, j * 32 + (i >> 2) * 8 + (i & 3))) - delta);
                     else
-                        ds[j][i] = p * fmaf(dp[j][i], 0.9f, -delta);
+                        ds[i] = p * fmaf(dp[i], 0.9f, -delta);
                 }
                 // as in the dK/dV pass: only a masked launch can have p != 0 on hidden elements
                 if (HAS_MASK && masked) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[j][i] = and_bits(ds[j][i], bit_mask(okbits[j], i));
+                    for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
                 }
                 if constexpr (HAS_MASK) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[j][i] = mask_select(ds[j][i], 0.f, mask_lanes(mwords, i));
+                    for (int i = 0; i < 16; ++i) ds[i] = mask_select(ds[i], 0.f, mask_lanes(mwords, i));
                 }
+                tp_x_regs_one(dq, base + 2 * X::NP * PANEL, ds, j, lr, lg, T());   // dQ^T += K^T dS^T
             }
-            tp_x_regs(dq, base + 2 * X::NP * PANEL, ds, lr, lg, T());    // dQ^T += K^T dS^T
         }
         __builtin_amdgcn_sched_barrier(0);
         DQ_STASH(st ^ 1)
