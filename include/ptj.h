@@ -261,7 +261,9 @@ int ptj_attn_fwd(const void* q, const void* k, const void* v, const uint32_t* ma
 
 /* Flash-attention backward with P recomputed from (ms, ls).  Outputs dq/dk/dv
  * [BH, T, dh] with explicit strides.  Deterministic: dK/dV and dQ are produced by
- * two passes, no atomics.  `workspace` (always required here) holds
+ * two passes, no atomics (the dQ pass runs first and leaves rowsum(dO*O) in the
+ * workspace for the dK/dV pass), so no output may overlap an input.  `workspace`
+ * (always required here) holds
  * ptj_attn_workspace_bytes(B, H, T) bytes.  Replaces
  * t_scaled_dot_prod_attn_bkwd3_k/_t (model_triton.py:829-1003). */
 int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, const void* o,

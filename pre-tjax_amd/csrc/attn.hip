@@ -55,7 +55,7 @@ struct AttnArgs {
     //   then the same amount:  word (b, k/32, q) holds M[b, q, 32*(k/32) + r] in bit r   (lane = key)
     const uint32_t* mask;
     float *ms, *ls;               // [BH, T]
-    const float* delta;           // [BH, T] rowsum(dO * O)  (backward)
+    float* delta;                 // [BH, T] rowsum(dO * O)  (backward: written by the dQ pass, read by the dK/dV pass)
     const uint32_t* keepbits;     // [BH, bitwords]  (train)
     int B, H, T, bitwords;
     // element strides: batch, head, row (the head dimension itself has unit stride)
@@ -265,36 +265,6 @@ __global__ __launch_bounds__(256) void attn_pack_mask_kernel(const uint8_t* __re
         }
         out[i] = w;
     }
-}
-
-// ---- delta[bh, q] = sum_d dO[q,d] * O[q,d] -------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
-                                                          float* __restrict__ delta, int T_, int H_,
-                                                          int64_t do_bs, int64_t do_hs, int64_t do_rs, int64_t o_bs,
-                                                          int64_t o_hs, int64_t o_rs) {
-    const int bh = blockIdx.y;
-    const int64_t do_off = (bh / H_) * do_bs + (bh % H_) * do_hs, o_off = (bh / H_) * o_bs + (bh % H_) * o_hs;
-    const int row = blockIdx.x * 32 + (threadIdx.x >> 3);
-    const int c = (threadIdx.x & 7) * 8;
-    float s = 0.f;
-    if (row < T_) {
-        const T* pa = d_o + do_off + (int64_t)row * do_rs + c;
-        const T* pb = o + o_off + (int64_t)row * o_rs + c;
-        constexpr int V = VecOf<T>::N;
-#pragma unroll
-        for (int h = 0; h < 8 / V; ++h) {
-            float x[V], y[V];
-            load_vec<T, V>(pa + h * V, x);
-            load_vec<T, V>(pb + h * V, y);
-#pragma unroll
-            for (int e = 0; e < V; ++e) s += x[e] * y[e];
-        }
-    }
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
-    s += __shfl_xor(s, 4, 64);
-    if ((threadIdx.x & 7) == 0 && row < T_) delta[(int64_t)bh * T_ + row] = s;
 }
 
 // ---- element-wise pieces (VALU budget: a wave64 VALU op costs 4 cycles, v_exp 16, and one
@@ -662,7 +632,22 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     const int64_t si = (int64_t)bh * a.T + qrow;
     // as in the dK/dV pass: 1/l folded into the exponent for 2-byte storage without a mask
     constexpr bool FOLD_L = sizeof(T) == 2 && !HAS_MASK;
-    const float linv = 1.0f / a.ls[si], delta = a.delta[si];
+    const float linv = 1.0f / a.ls[si];
+    // delta = rowsum(dO * O) of the lane's query: each lane of the pair (lr, lg) holds one half
+    // of the dO row already; the dK/dV pass (launched after this one) reads the stored values.
+    float delta;
+    {
+        typename X::F of[X::NC];
+        load_row_frags<T>(of, (const T*)a.o + bidx * a.o_bs + hidx * a.o_hs + (int64_t)qrow * a.o_rs, lg);
+        constexpr int FE = (int)(sizeof(typename X::F) / sizeof(T));
+        float part = 0.f;
+#pragma unroll
+        for (int c = 0; c < X::NC; ++c)
+#pragma unroll
+            for (int e = 0; e < FE; ++e) part += (float)dof[c][e] * (float)of[c][e];
+        delta = part + xor32(part);
+        if (lg == 0 && query < a.T) a.delta[si] = delta;
+    }
     const float m2 = FOLD_L ? fmaf(a.ms[si], LOG2E, __builtin_amdgcn_logf(a.ls[si])) : a.ms[si] * LOG2E;
 
     int nkt = (q0 + 128) / 64;
@@ -892,14 +877,6 @@ int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, c
         rc = launch_keepbits(bits, BH, a.bitwords, seed, st);
         if (rc) return rc;
     }
-    dim3 dgrid((unsigned)((T + 31) / 32), (unsigned)BH);
-    if (dtype == PTJ_F32)
-        hipLaunchKernelGGL((attn_delta_kernel<float>), dgrid, dim3(256), 0, st, (const float*)d_o, (const float*)o, delta,
-                           (int)T, (int)H, do_bs, do_hs, do_rs, o_bs, o_hs, o_rs);
-    else
-        hipLaunchKernelGGL((attn_delta_kernel<bf16>), dgrid, dim3(256), 0, st, (const bf16*)d_o, (const bf16*)o, delta,
-                           (int)T, (int)H, do_bs, do_hs, do_rs, o_bs, o_hs, o_rs);
-    PTJ_CHECK_LAUNCH();
     dim3 grid((unsigned)BH, (unsigned)((T + 127) / 128));
     AttnArgs a1 = a;
     a1.out0 = dk; a1.out0_bs = dk_bs; a1.out0_hs = dk_hs; a1.out0_rs = dk_rs;
@@ -907,11 +884,11 @@ int ptj_attn_bwd(const void* d_o, const void* q, const void* k, const void* v, c
     AttnArgs a2 = a;
     a2.out0 = dq; a2.out0_bs = dq_bs; a2.out0_hs = dq_hs; a2.out0_rs = dq_rs;
     if (dtype == PTJ_F32) {
-        ATTN_LAUNCH(attn_bwd_dkdv_kernel, float, grid, st, a1);
-        ATTN_LAUNCH(attn_bwd_dq_kernel, float, grid, st, a2);
+        ATTN_LAUNCH(attn_bwd_dq_kernel, float, grid, st, a2);      // also writes delta ...
+        ATTN_LAUNCH(attn_bwd_dkdv_kernel, float, grid, st, a1);    // ... which this pass reads
     } else {
-        ATTN_LAUNCH(attn_bwd_dkdv_kernel, bf16, grid, st, a1);
         ATTN_LAUNCH(attn_bwd_dq_kernel, bf16, grid, st, a2);
+        ATTN_LAUNCH(attn_bwd_dkdv_kernel, bf16, grid, st, a1);
     }
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
