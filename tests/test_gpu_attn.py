@@ -125,6 +125,38 @@ def test_attn_dropout_mask_bits(mt):
     assert torch.allclose(f64(o), want, rtol=1e-5, atol=1e-7)
 
 
+def test_attn_full_size_train_properties(mt):
+    """BASELINE config 5 shape (B16 H12 T1024, bf16, dropout on): properties that need no oracle.
+    (1) the backward is linear in dO, and a scaling by 2 commutes with every rounding, so
+        bwd(2 dO) == 2 bwd(dO) bit for bit -- which also holds only if the dK/dV pass reads the
+        row sums rowsum(dO*O) of THIS call (the dQ pass of the same call writes them);
+    (2) with v = 1 and dO = 1: O[q, :] = sum_k Pdrop[q, k] and dV[k, :] = sum_q Pdrop[q, k], so both
+        have the same grand total per batch-head -- forward and backward apply one dropout mask."""
+    B, H, T, seed = 16, 12, 1024, 99
+    g = gen(8)
+    q = randn(g, B, H, T, 64, dtype=torch.bfloat16).to(DEV)
+    k = randn(g, B, H, T, 64, dtype=torch.bfloat16).to(DEV)
+    v = randn(g, B, H, T, 64, dtype=torch.bfloat16).to(DEV)
+    dO = randn(g, B, H, T, 64, dtype=torch.bfloat16).to(DEV)
+    o, ms, ls = mt.attn_fwd_t(q, k, v, None, True, seed)
+    d1 = [t.clone() for t in mt.attn_bwd_t(dO, q, k, v, o, ms, ls, None, True, seed)]
+    d2 = mt.attn_bwd_t(dO * 2, q, k, v, o, ms, ls, None, True, seed)
+    for a, b, name in zip(d1, d2, ("dq", "dk", "dv")):
+        assert torch.equal(a * 2, b), name
+    again = mt.attn_bwd_t(dO, q, k, v, o, ms, ls, None, True, seed)
+    for a, b, name in zip(d1, again, ("dq", "dk", "dv")):
+        assert torch.equal(a, b), name + " not reproducible"
+
+    ones = torch.ones_like(v)
+    o1, ms1, ls1 = mt.attn_fwd_t(q, k, ones, None, True, seed)
+    _, _, dv1 = mt.attn_bwd_t(ones, q, k, ones, o1, ms1, ls1, None, True, seed)
+    tot_o = o1[..., 0].double().sum(dim=-1)          # [B, H]
+    tot_dv = dv1[..., 0].double().sum(dim=-1)
+    assert torch.allclose(tot_o, tot_dv, rtol=2e-3), (tot_o - tot_dv).abs().max().item()
+    # about a tenth of the probability mass is dropped
+    assert 0.85 * T < tot_o.mean().item() < 0.95 * T
+
+
 def test_attn_strided_views_fused_qkv_layout(mt):
     # q/k/v as column slices of one [B*T, H*3*dh] buffer, O written into [B,T,H*dh]
     B, H, T = 2, 4, 128
