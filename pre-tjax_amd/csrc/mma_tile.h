@@ -66,13 +66,18 @@ struct TileLoader {
     // KMAJOR / GENERIC geometry
     static constexpr int RP = THREADS / 8;          // rows per pass (8 threads cover one 128-byte row)
     static constexpr int NV = (ROWS + RP - 1) / RP; // vectors per thread
-    // MNMAJOR geometry: a block = 8 row-vectors x 8 quads = one wave-wide instruction
-    static constexpr int JB = ROWS / VEC / 8;       // blocks along rows
-    static constexpr int KB = BK / 4 / 8;           // blocks along k (bf16: 2, fp32: 1)
+    // MNMAJOR geometry: a block = RB row-vectors x QB quads = one wave-wide instruction.  QB
+    // quads span a whole 128-byte panel row (2-byte elements: 16 quads of 8 bytes, 4-byte: 8
+    // quads of 16 bytes), so one LDS store instruction writes RB complete rows -- every bank
+    // equally often, whatever the swizzle.
+    static constexpr int QB = BK / 4;               // quads of one block along k: 16 / 8
+    static constexpr int RB = 64 / QB;              // row vectors of one block: 4 / 8
+    static constexpr int JB = ROWS / VEC / RB;      // blocks along rows
+    static constexpr int KB = 1;                    // blocks along k
     static constexpr int NBLK = JB * KB;
     static constexpr int NW = THREADS / 64;
     static constexpr int NQ = (NBLK + NW - 1) / NW; // quads per thread
-    static_assert(ROWS % (VEC * 8) == 0 && BK % 32 == 0, "panel shape");
+    static_assert(ROWS % (VEC * RB) == 0 && BK % 32 == 0, "panel shape");
     static constexpr int NREG = MODE == MNMAJOR ? NQ * 4 : NV;
     u32x4 r[NREG];
 
@@ -124,19 +129,19 @@ struct TileLoader {
                 }
             }
         } else {
-            const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
+            const int jc_lo = tid & (RB - 1), kq_lo = (tid & 63) / RB, w = tid >> 6;
             const char* ub = reinterpret_cast<const char*>(p + (int64_t)k0 * s_k + (CLAMP ? 0 : row0));   // uniform
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
                 if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
-                    int rowv = ((b % JB) * 8 + jc_lo) * VEC;               // first row of the lane's row vector
+                    int rowv = ((b % JB) * RB + jc_lo) * VEC;              // first row of the lane's row vector
                     if constexpr (CLAMP) {
                         const int lastv = ((nrows - 1) / VEC) * VEC;        // a .t() view's pitch covers this vector
                         rowv = row0 + rowv < lastv ? row0 + rowv : lastv;
                     }
                     const uint32_t loff =
-                        ((uint32_t)(((b / JB) * 8 + kq_lo) * 4) * (uint32_t)s_k + (uint32_t)rowv) * (uint32_t)sizeof(T);
+                        ((uint32_t)(((b / JB) * QB + kq_lo) * 4) * (uint32_t)s_k + (uint32_t)rowv) * (uint32_t)sizeof(T);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         if ((qi * 4 + i) % N != I) continue;
@@ -166,12 +171,12 @@ struct TileLoader {
                 r[i] = v;
             }
         } else {
-            const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
+            const int jc_lo = tid & (RB - 1), kq_lo = (tid & 63) / RB, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
-                const int row = row0 + ((b % JB) * 8 + jc_lo) * VEC;
-                const int kq = k0 + ((b / JB) * 8 + kq_lo) * 4;
+                const int row = row0 + ((b % JB) * RB + jc_lo) * VEC;
+                const int kq = k0 + ((b / JB) * QB + kq_lo) * 4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     u32x4 v = {0u, 0u, 0u, 0u};
@@ -201,13 +206,13 @@ struct TileLoader {
                     *reinterpret_cast<u32x4*>(lds + row * BKB + ((c ^ sw(row)) << 4)) = r[i];
             }
         } else {
-            const int jc_lo = tid & 7, kq_lo = (tid >> 3) & 7, w = tid >> 6;
+            const int jc_lo = tid & (RB - 1), kq_lo = (tid & 63) / RB, w = tid >> 6;
 #pragma unroll
             for (int qi = 0; qi < NQ; ++qi) {
                 const int b = WRAP ? (w + qi * NW) % NBLK : w + qi * NW;
                 if (WRAP || (NBLK % NW == 0) || (b < NBLK)) {
-                    const int prow = ((b % JB) * 8 + jc_lo) * VEC;
-                    int kq = (b / JB) * 8 + kq_lo;
+                    const int prow = ((b % JB) * RB + jc_lo) * VEC;
+                    int kq = (b / JB) * QB + kq_lo;
                     if constexpr (PAIRQ && sizeof(T) == 2) kq = (kq & ~3) | ((kq & 1) << 1) | ((kq >> 1) & 1);
                     const int kb = kq * 4 * (int)sizeof(T);  // byte offset of the quad in the row
 #pragma unroll
