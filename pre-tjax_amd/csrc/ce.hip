@@ -92,7 +92,7 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
     constexpr bool LAND = CACHED && sizeof(T) == 2;
     __shared__ __attribute__((aligned(16))) char land[LAND ? CE_THREADS * ITERS * 16 : 16];
     __shared__ float smem[16];
-    __shared__ int smin[16];
+    __shared__ int s_best;
     __shared__ float s_xy;
     const float inv_cnt = 1.0f / (float)(*count);
     if constexpr (LAND) {
@@ -108,6 +108,7 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
         const int nvec = (cols + mis + VEC - 1) / VEC;
         const int64_t label = labels[row];
         if (t == 0 && label != 0) s_xy = to_f32(xr[label]);  // read before any in-place write
+        if (t == 0) s_best = 0x7fffffff;   // ordered before this row's candidates by the max reduction's barrier
 
         float v[ITERS][VEC];
         float m = -INFINITY;
@@ -189,10 +190,9 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                     }
                 }
             }
-            best = wave_min_int(best);
-            // per-wave results; folded by thread 0 after the barriers of the sum reduction below
-            // (the next write happens behind the next row's max reduction, which synchronises too)
-            if ((t & 63) == 0) smin[t >> 6] = best;
+            // the few threads that hold the maximum post their lowest column; thread 0 reads the
+            // result after the barriers of the sum reduction below
+            if (best != 0x7fffffff) atomicMin(&s_best, best);
         }
         float s = 0.f;
         if constexpr (CACHED) {
@@ -216,11 +216,7 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
         }
         s = row_reduce<CE_THREADS, false>(s, smem);  // contains __syncthreads: s_xy is visible after it
         const bool live = label != 0;
-        if (t == 0 && pred != nullptr) {
-            int b = smin[0];
-            for (int i = 1; i < CE_THREADS / 64; ++i) b = smin[i] < b ? smin[i] : b;
-            pred[row] = b;
-        }
+        if (t == 0 && pred != nullptr) pred[row] = s_best;
         if (t == 0) row_loss[row] = live ? -(s_xy - m - logf(s)) : 0.f;
         const float scale = live ? inv_cnt / s : 0.f;
 
