@@ -11,7 +11,8 @@
 // with the same trick mirrored: a lane owns one key, dV^T = dO^T P and dK^T = Q^T dS.
 // The operand that must be read "across" its memory layout (V^T, K^T, Q^T, dO^T: row
 // index d, contraction along keys / queries) is transposed once while it is written to
-// LDS (MNMAJOR panel loader) and shared by the four wavefronts.
+// LDS (MNMAJOR panel loader, quads paired so that the eight positions a lane holds of an
+// accumulator tile are one 16-byte chunk) and shared by the four wavefronts.
 //
 // Softmax is evaluated in base 2 (scores pre-multiplied by log2(e)/sqrt(dh)); the saved
 // statistics `ms` are converted back to natural units.  Masked scores take the
@@ -22,8 +23,9 @@
 // one line of 2T keep bits per batch-head is generated once (attn_keepbits_kernel); the
 // kernels read it through the scalar unit and turn it into 64-lane select masks.
 //
-// The backward is two passes without atomics: (dK, dV) over key tiles, dQ over query
-// tiles; both recompute S and dP.
+// The backward is two passes without atomics: dQ over query tiles (it also forms
+// delta = rowsum(dO * O) of its queries and stores it), then (dK, dV) over key tiles,
+// which reads delta; both recompute S and dP.
 #include "common.h"
 #include "mma_tile.h"
 
