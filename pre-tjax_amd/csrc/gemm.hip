@@ -698,16 +698,41 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const GemmArgs g)
     int row0, col0;
     tile_origin(g.tail_first + t, num_m * num_n, num_m, num_n, row0, col0);
     const float* base = g.partial + (int64_t)t * g.tail_splits * (BM * BN);
-    for (int i = blockIdx.y * 256 + threadIdx.x; i < BM * BN; i += gridDim.y * 256) {
+    // four consecutive columns per thread: 16-byte loads of the partial tiles; a quad that lies
+    // wholly inside C is stored as one vector when the outputs allow it
+    for (int q = blockIdx.y * 256 + threadIdx.x; q < BM * BN / 4; q += gridDim.y * 256) {
+        const int i = q * 4;
         const int r = i / BN, c = i - r * BN;
         const int row = row0 + r, col = col0 + c;
         if (row >= g.n || col >= g.m) continue;
-        float s = 0.f;
-        for (int z = 0; z < g.tail_splits; ++z) s += base[(int64_t)z * (BM * BN) + i];
-        if (g.epilogue != PTJ_EPI_NONE) s += to_f32(((const T*)g.bias)[col]);
-        if (g.c_aux != nullptr) ((T*)g.c_aux)[(int64_t)row * g.c_aux_rs + col] = from_f32<T>(s);
-        if (g.epilogue == PTJ_EPI_BIAS_GELU) s = gelu_f(s);
-        ((T*)g.c)[(int64_t)row * g.c_rs + col] = from_f32<T>(s);
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int z = 0; z < g.tail_splits; ++z) s += *reinterpret_cast<const f32x4*>(base + (int64_t)z * (BM * BN) + i);
+        const bool whole = col + 4 <= g.m;
+        if (g.epilogue != PTJ_EPI_NONE) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (whole || col + e < g.m) s[e] += to_f32(((const T*)g.bias)[col + e]);
+        }
+        T* ca = g.c_aux != nullptr ? (T*)g.c_aux + (int64_t)row * g.c_aux_rs + col : nullptr;
+        T* cc = (T*)g.c + (int64_t)row * g.c_rs + col;
+        Pack<T, 4> pre, out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            pre.v[e] = from_f32<T>(s[e]);
+            out.v[e] = from_f32<T>(g.epilogue == PTJ_EPI_BIAS_GELU ? gelu_f(s[e]) : s[e]);
+        }
+        if (whole && g.vec_out) {
+            if (ca != nullptr) *reinterpret_cast<Pack<T, 4>*>(ca) = pre;
+            *reinterpret_cast<Pack<T, 4>*>(cc) = out;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (col + e >= g.m) break;
+                if (ca != nullptr) ca[e] = pre.v[e];
+                cc[e] = out.v[e];
+            }
+        }
     }
 }
 
