@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 # Measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this benchmark (commands, per-kernel table
 # and the copy-kernel scale factors: profiles/hbm_traffic__gpt2_b16_t1024_bf16_step.md): 228.3e6 read +
 # 69.3e6 written per GEMM launch, averaged over the forward, dX and dW products of a step.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 237.7e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 237.9e6
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
