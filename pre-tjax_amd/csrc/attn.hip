@@ -300,7 +300,8 @@ __device__ __forceinline__ int32_t bit_mask(uint32_t w, int pos) { return __buil
 // ---- forward -------------------------------------------------------------------------
 // grid (B*H, ceil(T/128)); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
 template <typename T, bool HAS_MASK, bool TRAIN>
-__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
+// (2-byte storage: three workgroups per CU = three wavefronts per SIMD, 168 registers each)
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 2 * X::NP * PANEL;  // K panels then V^T panels
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
@@ -610,7 +611,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 // ---- backward pass 2: dQ ----------------------------------------------------------------
 // Same geometry as the forward (lane = query, key tiles of 64).
 template <typename T, bool HAS_MASK, bool TRAIN>
-__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
+// (2-byte storage without an explicit mask fits three wavefronts per SIMD; the bound keeps it there)
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 3 * X::NP * PANEL;  // K, V, K^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
