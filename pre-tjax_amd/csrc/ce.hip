@@ -171,13 +171,14 @@ __global__ __launch_bounds__(1024) void ce_row_kernel(const int64_t* __restrict_
                 // only a thread that holds the maximum searches for its position (typically one
                 // thread of the row; the others skip the scan)
                 if (m_own == m) {
+                    // from the thread's last element down to its first, so the lowest match is the
+                    // one that stays: a compare and a select on a constant per element
+                    int off = 0x7fffffff;
 #pragma unroll
-                    for (int it = 0; it < ITERS; ++it)
+                    for (int it = ITERS - 1; it >= 0; --it)
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            const int e = (t + it * CE_THREADS) * VEC + j - mis;
-                            if (v[it][j] == m && e < best) best = e;
-                        }
+                        for (int j = VEC - 1; j >= 0; --j) off = v[it][j] == m ? it * CE_THREADS * VEC + j : off;
+                    if (off != 0x7fffffff) best = off + t * VEC - mis;
                 }
             } else {
                 for (int vi = t; vi < nvec; vi += CE_THREADS) {
