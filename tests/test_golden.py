@@ -68,6 +68,28 @@ def test_gpu_dropout_masks_equal_golden(mt, gold):
 
 
 @pytest.mark.gpu
+def test_gpu_dropout_masks_equal_triton_package_values(mt):
+    """Keep decisions written by the installed Triton package's own tl.rand
+    (tests/golden/make_tl_rand.py), row-wise and attention addressing, all four seeds."""
+    with np.load(os.path.join(HERE, "golden", "tl_rand_v1.npz"), allow_pickle=False) as z:
+        fx = {k: z[k] for k in z.files}
+    for seed in fx["seeds"].tolist():
+        want = torch.from_numpy(fx["rows_keep_%d" % seed])
+        for dtype in (torch.float32, torch.bfloat16):
+            got = mt.t_dropout_fwd_t(torch.ones(want.shape, dtype=dtype, device=DEV), True, seed)
+            assert torch.equal(got.cpu() != 0, want), seed
+        # attention: the fixture covers q, k < 16; V = identity shows the kept probabilities
+        want = torch.from_numpy(fx["attn_keep_%d" % seed])                  # [3, 16, 16]
+        B, H, T, dh = 1, want.shape[0], 64, 64
+        z4 = torch.zeros(B, H, T, dh, device=DEV)
+        v = torch.eye(T, dh, device=DEV).expand(B, H, T, dh).contiguous()
+        o, _, _ = mt.attn_fwd_t(z4, z4.clone(), v, None, True, seed)
+        n = want.shape[1]
+        tril = torch.tril(torch.ones(n, n, dtype=torch.bool))
+        assert torch.equal((o[0, :, :n, :n].cpu() != 0) & tril, want & tril), seed
+
+
+@pytest.mark.gpu
 def test_gpu_attention_dropout_mask_equals_golden(mt, gold):
     # V = identity padded to dh columns makes row q of O the dropped probabilities of q: the
     # zero pattern below the diagonal is the keep mask (seed + batch-head, offset q + k)

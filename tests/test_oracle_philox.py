@@ -66,3 +66,31 @@ def test_attn_mask_depends_on_q_plus_k_only():
     q, k = np.meshgrid(np.arange(8), np.arange(8), indexing="ij")
     line = philox.tl_rand(np.int64(3 + 1), np.arange(15)) > np.float32(0.1)
     assert (m[1] == line[q + k]).all()
+
+
+def _tl_rand_fixture():
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tl_rand_v1.npz")
+    return np.load(path)
+
+
+def test_tl_rand_matches_the_triton_package():
+    """oracle.philox against values written by the installed Triton package's own tl.rand
+    (tests/golden/make_tl_rand.py): the seed -> key split, the offset -> counter word, the
+    choice of output word 0 and the float fold are all fixed by these, bit for bit."""
+    fx = _tl_rand_fixture()
+    for s in fx["seeds"].tolist():
+        rows_u = fx["rows_u_%d" % s]
+        n_rows, n_cols = rows_u.shape
+        got = philox.tl_rand(np.arange(n_rows, dtype=np.int64)[:, None] + np.int64(s),
+                             np.arange(n_cols, dtype=np.int64)[None, :])
+        assert got.dtype == np.float32 and (got.view(np.uint32) == rows_u.view(np.uint32)).all(), s
+        assert (philox.rowwise_keep_mask(s, n_rows, n_cols) == fx["rows_keep_%d" % s]).all(), s
+        attn_keep = fx["attn_keep_%d" % s]
+        bh, tq, tk = attn_keep.shape
+        assert (philox.attn_keep_mask(s, bh, tq, tk) == attn_keep).all(), s
+        q, k = np.meshgrid(np.arange(tq), np.arange(tk), indexing="ij")
+        u = philox.tl_rand(np.arange(bh, dtype=np.int64)[:, None, None] + np.int64(s), (q + k)[None])
+        assert (u.view(np.uint32) == fx["attn_u_%d" % s].view(np.uint32)).all(), s
+    # the fixture exercises both decisions
+    assert not fx["rows_keep_42"].all() and fx["rows_keep_42"].any()
