@@ -56,7 +56,7 @@ def make_state(torch, lo, c, dev):
                        rn(D, F, scale=res), torch.zeros(D, device=dev)])
     master.append([torch.ones(D, device=dev), torch.zeros(D, device=dev)])
     shadow = [[p.to(torch.bfloat16) for p in grp] for grp in master]
-    moments = lo.init_adam_w(master)
+    _, moments = lo.init_adam_w(master)
     # weight decay on matrices only (train_gpt2_triton.py:71: not the 1-D zero-initialised tensors)
     wd_mask = [[p.dim() > 1 for p in grp] for grp in master]
     return master, shadow, moments, wd_mask
@@ -94,7 +94,7 @@ def main():
     seed_gen = torch.Generator().manual_seed(100)
     n_total = args.warmup + 2 * args.steps
     tokens = torch.randint(0, V, (n_total, B, T + 1), generator=tok_gen).to(dev)
-    mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=dev)).expand(B, T, T)
+    mask = None   # plain causal mask (unpadded, unpacked synthetic sequences): masked by index in the kernels
     seeds = [lo.sample_p_gen_aux(master, seed_gen) for _ in range(n_total)]
     losses = []
 

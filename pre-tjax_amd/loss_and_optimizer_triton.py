@@ -1,11 +1,13 @@
 """Loss-side wrappers with the reference's names (loss_and_optimizer_triton.py of
 martin-kukla/pre-tjax) on top of libptj.so."""
 import ctypes
+import math
 
 import torch
 
 from ._lib import check, dtype_code, lib, ptr, require_gpu, stream
 from .model_triton import _workspace
+from .spec_torch import accuracy, t_avg_cross_entropy_loss, t_avg_cross_entropy_loss_bkwd3  # noqa: F401  (torch twins)
 
 
 def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Tensor, inplace=False, want_pred=False):
@@ -68,17 +70,68 @@ def sample_p_gen_aux(params, generator=None):
     return torch.randint(0, 1_000_000, (n,), generator=generator).tolist()
 
 
+def t_acc_grad_loss3_t(acc_grads, params, y, y_mask, y_indices):
+    """One micro-step of gradient accumulation on the kernel path
+    (loss_and_optimizer_triton.py:336-337): -> (acc_grads, (loss, acc, non-pad fraction))."""
+    return _acc_grad_loss(t_loss_bkwd3_t, acc_grads, params, y, y_mask, y_indices)
+
+
+def _acc_grad_loss(grad_loss_fn, acc_grads, params, y, y_mask, y_indices):
+    """loss_and_optimizer_triton.py:340-348: fresh dropout seeds, one forward+backward, and
+    the step's gradients added onto `acc_grads` (entries are rebound, as in the reference;
+    the sums are formed in the accumulator's dtype by multi-tensor adds, a few launches for
+    the whole nest)."""
+    step_grads, rest = grad_loss_fn(params, y, y_mask, y_indices, train=True, p_gen_aux=sample_p_gen_aux(params))
+    flat_acc = [a for grp in acc_grads for a in grp]
+    flat_new = [g.to(a.dtype).reshape(a.shape) for grp_a, grp_g in zip(acc_grads, step_grads)
+                for a, g in zip(grp_a, grp_g)]
+    summed = iter(torch._foreach_add(flat_acc, flat_new))
+    for grp in acc_grads:
+        for pi in range(len(grp)):
+            grp[pi] = next(summed)
+    return acc_grads, rest
+
+
+def _sq_norms(tensors):
+    return [n * n for n in torch._foreach_norm([t.float() for t in tensors])]
+
+
+def grads_l2norm(grads):
+    """Global L2 norm of a gradient nest as a Python float (reference :411-414)."""
+    return math.sqrt(float(torch.stack(_sq_norms([g for grp in grads for g in grp])).sum()))
+
+
+def grads_grps_l2norms(grads):
+    """Per-group L2 norms of a gradient nest as Python floats (reference :415-416)."""
+    return [math.sqrt(float(torch.stack(_sq_norms(list(grp))).sum())) for grp in grads]
+
+
+def elwise(params_and_grads, func):
+    """Apply `func` leaf by leaf over nests of equal shape (reference :355-356)."""
+    return [[func(*leaves) for leaves in zip(*groups)] for groups in zip(*params_and_grads)]
+
+
+def sgd(params, grads, lr):
+    """reference :358-359."""
+    return elwise((params, grads), lambda p, g: p - lr * g)
+
+
 def init_adam_w(params):
-    """fp32 first/second moments shaped like `params` (reference :362-363)."""
-    return [[[torch.zeros_like(p, dtype=torch.float32) for p in grp] for grp in params] for _ in range(2)]
+    """(zero gradient accumulators, [first moments, second moments]), each shaped like
+    `params` (loss_and_optimizer_triton.py:362-363).  The moments are fp32 whatever the
+    parameter dtype; the accumulators take the parameters' dtype."""
+    zeros = lambda dt: [[torch.zeros_like(p, dtype=dt or p.dtype) for p in grp] for grp in params]
+    return zeros(None), [zeros(torch.float32), zeros(torch.float32)]
 
 
-def adam_w_in_place(master, grads, lr, betas, epsilon, moments, i, weight_decay=0.0, weight_decay_mask=None,
+def adam_w_in_place(params, grads, lr, betas, epsilon, moments, i, weight_decay=0.0, weight_decay_mask=None,
                     shadow=None):
     """AdamW of the reference (:376-401: t = i+1, bias-corrected moments, decay scaled by
     lr) on fp32 master weights: one fused HIP pass over the whole nest (a few launches)
     instead of ~10 torch ops per tensor.
-    `shadow` (optional nest of low-precision copies) is refreshed from the masters."""
+    `params` are the fp32 master weights, updated in place; `shadow` (optional nest of
+    low-precision copies) is refreshed from them."""
+    master = params
     t = i + 1
     ps, ms_, vs, gs, ss, ns, wds = [], [], [], [], [], [], []
     keep = []                                    # contiguous gradient copies must outlive the launch

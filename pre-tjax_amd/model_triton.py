@@ -12,6 +12,13 @@ import torch
 
 from . import _lib
 from ._lib import check, dtype_code, lib, ptr, require_gpu, stream
+# plain-torch twins of the wrappers (the reference's names without `_t`); not used below
+# except `t_gelu_fwd`, which callers pass as the `activation_fn` marker
+from .spec_torch import (t_dropout_bkwd2, t_dropout_fwd, t_gelu_bkwd2, t_gelu_fwd,  # noqa: F401
+                         t_layernorm_bkwd2_p, t_layernorm_bkwd2_x, t_layernorm_fwd, t_linear_fwd,
+                         t_log_softmax_bkwd2, t_log_softmax_fwd, t_proj_fwd, t_scaled_dot_prod_attn_bkwd3,
+                         t_scaled_dot_prod_attn_fwd, t_scaled_dot_prod_attn_fwd3, t_softmax_attn_fwd,
+                         t_tlayer_ffn_fwd)
 
 DROPOUT_RATE = 0.1  # baked into the kernels, as in the reference (model_torch_func.py:2)
 
@@ -19,9 +26,9 @@ _ws_cache = {}
 
 
 def _workspace(nbytes, device, tag):
-    """Reusable scratch buffer per (device, tag); grown on demand.  Kernels that use it
-    are ordered on one stream, so sharing between consecutive calls is safe."""
-    key = (device, tag)
+    """Reusable scratch buffer per (device, stream, tag); grown on demand.  Kernels that use
+    it are ordered on one stream, so sharing between consecutive calls is safe."""
+    key = (device, stream(), tag)
     buf = _ws_cache.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
@@ -321,14 +328,9 @@ def t_matmul_t(a: torch.Tensor, b: torch.Tensor):
 t_matmul = t_matmul_t
 
 
-def t_gelu_fwd(x):
-    """Marker for `activation_fn` arguments (the reference passes its torch GELU here,
-    model_triton.py:221); evaluating it runs the HIP kernel."""
-    return t_gelu_fwd_t(x)
-
-
 def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
-    """Two GEMM launches: bias+GELU epilogue, then bias (model_triton.py:1258-1313)."""
+    """Two GEMM launches: bias+GELU epilogue, then bias (model_triton.py:1258-1313).
+    `activation_fn` is the reference's marker argument: its torch GELU (`t_gelu_fwd`)."""
     assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU epilogue exists"
     w1, b1, w2, b2 = layer_params
     shape = x.shape
@@ -338,6 +340,26 @@ def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
     return out.view(shape[:-1] + (w2.shape[0],))
 
 
+def t_tlayer_ffn_bkwd2_t(dloss_dx, layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
+    """VJP of the feed-forward block without saved activations (model_triton.py:1410-1428):
+    the first linear layer is recomputed (bias+GELU epilogue that also keeps the
+    pre-activation), then dW2, db2, d(mid), GELU backward with db1, dW1 and dx.
+    Returns (dx shaped like x, (dW1, db1, dW2, db2))."""
+    assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU backward exists"
+    w1, b1, w2, b2 = layer_params
+    x2 = _rows2d(x)
+    d2 = _rows2d(dloss_dx)
+    pre = torch.empty((x2.shape[0], w1.shape[0]), dtype=x2.dtype, device=x2.device)
+    mid = matmul_t(x2, w1.t(), b1, gelu=True, pre_out=pre)
+    db2 = colsum_t(d2)
+    dw2 = matmul_t(d2.t(), mid)
+    dmid = matmul_t(d2, w2)
+    dpre, db1 = t_gelu_bkwd2_colsum_t(dmid, pre)
+    dw1 = matmul_t(dpre.t(), x2)
+    dx = matmul_t(dpre, w1)
+    return dx.reshape(x.shape), (dw1, db1, dw2, db2)
+
+
 # ----------------------------------------------------------------------------------
 # attention  (reference: model_triton.py:706-754 fwd3_t, :951-1003 bkwd3_t)
 # ----------------------------------------------------------------------------------
@@ -345,32 +367,29 @@ _mask_cache = {}
 
 
 def _mask_arg(mask, B, T):
-    """None when `mask` is exactly the causal (lower-triangular) mask -- the kernel then
-    masks by index -- else the mask bit-packed for the kernels (ptj_attn_pack_mask).  The comparison reads the
-    mask once per distinct tensor (one host sync) and is cached on (address, version, layout).
-    A cache entry keeps its mask tensor alive: the address of a cached mask can therefore
-    not be handed to another tensor while the entry exists (a freed mask's address showing
-    up again under a different mask would otherwise be taken for the old one)."""
+    """The attention kernels' mask argument.  ``mask=None`` is the plain causal mask: the
+    kernels then mask by index.  Any tensor is bit-packed on the device for the kernels
+    (ptj_attn_pack_mask, both orientations) and applied as ``mask AND (key <= query)``; no
+    host comparison, no synchronisation.  The packed words are cached for the tensor they
+    were made from (address, version, layout, stream), so the 2L attention calls of a step
+    that share one mask pack it once; at most two entries live, each keeping its mask tensor
+    alive so that its address cannot be reused while the entry exists."""
     if mask is None:
         return None
     assert mask.shape[-2:] == (T, T), mask.shape
-    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device, B, T)
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device, B, T,
+           stream())
     hit = _mask_cache.get(key)
     if hit is None:
         m = mask.expand(B, T, T) if mask.dim() == 3 else mask.reshape(1, T, T).expand(B, T, T)
-        tril = torch.ones(T, T, dtype=torch.bool, device=mask.device).tril_()
-        if bool((m.to(torch.bool) == tril).all()):
-            hit = ("causal", None, mask)
-        else:
-            # bit-packed once per mask tensor, in the two orientations the kernels read
-            bytes_ = m.to(torch.bool).contiguous().view(torch.uint8)
-            packed = torch.empty(lib().ptj_attn_packed_mask_bytes(B, T) // 4, dtype=torch.int32, device=mask.device)
-            check(lib().ptj_attn_pack_mask(ptr(bytes_), ptr(packed), B, T, stream()), "ptj_attn_pack_mask")
-            hit = ("mask", packed, mask)
-        if len(_mask_cache) >= 8:
-            _mask_cache.clear()
+        bytes_ = m.to(torch.bool).contiguous().view(torch.uint8)
+        packed = torch.empty(lib().ptj_attn_packed_mask_bytes(B, T) // 4, dtype=torch.int32, device=mask.device)
+        check(lib().ptj_attn_pack_mask(ptr(bytes_), ptr(packed), B, T, stream()), "ptj_attn_pack_mask")
+        hit = (packed, mask)
+        while len(_mask_cache) >= 2:
+            _mask_cache.pop(next(iter(_mask_cache)))
         _mask_cache[key] = hit
-    return hit[1]
+    return hit[0]
 
 
 def _bhr(t):
@@ -540,10 +559,11 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None, h1=N
     return x_out.view(B, T, D), acts
 
 
-def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, mask, train=True, p_gen_aux=None, dropped_in=None,
+def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, y, mask, train=True, p_gen_aux=None, *, dropped_in=None,
                           drop_out=None, db2_in=None, drop_out_sum=False):
     """Backward of one block (model_triton.py:2291-2299 and the sub-block VJPs :2021-2039,
-    :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order).
+    :2175-2193).  dloss_dx [N,D] -> (dx [N,D], grads in parameter order).  `y` is the block's
+    input, in the reference's argument position; `acts` already holds it, so it is not read.
 
     `dropped_in`, if given, is t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2]) already
     computed by the producer of dloss_dx; `drop_out=(train, seed)` asks for the same service
@@ -666,7 +686,8 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
                                                        drop=(train, p_gen_aux[0]))
     layer_grads = [None] * L
     for i in reversed(range(L)):
-        res = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], y_mask, train, p_gen_aux[1 + 3 * i:4 + 3 * i],
+        res = t_gpt2_tlayer_bkwd3_t(dx, layer_acts[i], params[2 + i], layer_acts[i][0], y_mask, train,
+                                    p_gen_aux[1 + 3 * i:4 + 3 * i],
                                     dropped_in=dropped, db2_in=dsum,
                                     drop_out=(train, p_gen_aux[3 * i], layer_acts[i - 1][-1] if i > 0 else None),
                                     drop_out_sum=i > 0)

@@ -30,33 +30,39 @@ def make(B, H, T, dtype, seed=0):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("B,H,T", [(1, 1, 64), (2, 3, 128), (1, 2, 192), (2, 2, 256), (1, 12, 512)])
 @pytest.mark.parametrize("train", [False, True])
-def test_attn_fwd_bwd_causal(mt, dtype, B, H, T, train):
+@pytest.mark.parametrize("mask_as", ["tensor", "none"])
+def test_attn_fwd_bwd_causal(mt, dtype, B, H, T, train, mask_as):
+    """`tensor`: the lower-triangular mask as a bool tensor (bit-packed on the device, applied
+    from the packed words); `none`: mask=None, the kernels' index-masked causal path."""
     qkv, dO, mask = make(B, H, T, dtype, seed=T + B)
     seed = 4242
-    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), train, seed)
+    dmask = mask.to(DEV) if mask_as == "tensor" else None
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), dmask, train, seed)
     want_o = ops.scaled_dot_prod_attn_fwd(f64(qkv), mask, train, seed)
     close(o, want_o, dtype, "O")
     ms, ls = ops.scaled_dot_prod_attn_stats(f64(qkv), mask)
     assert acts[2] is o and acts[0].shape == (B, H, T)
     close(acts[0], ms, torch.float32 if dtype == torch.float32 else dtype, "ms")
     close(acts[1], ls, torch.float32 if dtype == torch.float32 else dtype, "ls")
-    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), dmask, train, seed)
     wq, wk, wv = ops.scaled_dot_prod_attn_bkwd(f64(dO), f64(qkv), mask, train, seed)
     close(dq, wq, dtype, "dq")
     close(dk, wk, dtype, "dk")
     close(dv, wv, dtype, "dv")
     # deterministic (no atomics)
-    dq2, dk2, dv2 = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    dq2, dk2, dv2 = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), dmask, train, seed)
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attn_config2_shape(mt, dtype):
+@pytest.mark.parametrize("mask_as", ["tensor", "none"])
+def test_attn_config2_shape(mt, dtype, mask_as):
     # BASELINE config 2: B=8, H=12, T=1024, dh=64 (oracle on a 2-batch slice to bound CPU time)
     B, H, T = 8, 12, 1024
     qkv, dO, mask = make(B, H, T, dtype, seed=2)
-    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), False)
-    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), False)
+    dmask = mask.to(DEV) if mask_as == "tensor" else None
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), dmask, False)
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), dmask, False)
     sl = slice(6, 8)
     want_o = ops.scaled_dot_prod_attn_fwd(f64(qkv[sl]), mask[sl], False)
     close(o[sl], want_o, dtype, "O")
@@ -91,23 +97,31 @@ def test_attn_padding_mask(mt, dtype, train):
     close(dv, wv, dtype, "dv")
 
 
-def test_attn_mask_detection_survives_address_reuse(mt):
-    """A causal mask is recognised once per tensor and cached; a different mask that later
-    lives at the address of a freed causal mask must not be taken for it."""
+def test_attn_fresh_mask_tensor_every_call(mt):
+    """The collator builds a new mask every batch: each call below gets a mask tensor that did
+    not exist before, alternating between two contents, so that a freed mask's address is
+    likely handed to a tensor with other content.  Nothing may be carried over from the
+    previous tensor at that address, and no call may need the host (the packed words are
+    made on the device from the tensor given)."""
     B, H, T = 2, 2, 256
     qkv, _, tril = make(B, H, T, torch.float32, seed=3)
     qd = qkv.to(DEV)
-    for _ in range(4):
-        m = tril.to(DEV)
-        o_causal, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m, False, 0)
+    padded = tril.clone()
+    padded[:, 128:, :128] = False
+    want = {"tril": ops.scaled_dot_prod_attn_fwd(f64(qkv), tril, False, 0),
+            "padded": ops.scaled_dot_prod_attn_fwd(f64(qkv), padded, False, 0)}
+    for it in range(8):
+        name, host = (("tril", tril), ("padded", padded))[it % 2]
+        m = host.to(DEV)                                 # a fresh device tensor
+        o, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m, False, 0)
+        close(o, want[name], torch.float32, "O %s call %d" % (name, it))
         del m                                            # its memory may be handed out again
-        padded = tril.clone()
-        padded[:, 128:, :128] = False
-        m2 = padded.to(DEV)
-        o_pad, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m2, False, 0)
-        close(o_causal, ops.scaled_dot_prod_attn_fwd(f64(qkv), tril, False, 0), torch.float32, "O causal")
-        close(o_pad, ops.scaled_dot_prod_attn_fwd(f64(qkv), padded, False, 0), torch.float32, "O padded")
-        del m2
+    # a mask rewritten in place (same address, new version) is packed again
+    m = tril.to(DEV)
+    mt.t_scaled_dot_prod_attn_fwd3_t(qd, m, False, 0)
+    m.copy_(padded.to(DEV))
+    o, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qd, m, False, 0)
+    close(o, want["padded"], torch.float32, "O after in-place rewrite")
 
 
 def test_attn_dropout_mask_bits(mt):
@@ -167,8 +181,7 @@ def test_attn_strided_views_fused_qkv_layout(mt):
     out = torch.empty(B, T, H * 64, dtype=torch.bfloat16, device=DEV)
     o, ms, ls = mt.attn_fwd_t(q, k, v, None, False, 0, out=out.view(B, T, H, 64).permute(0, 2, 1, 3))
     qkv = torch.stack((q, k, v), dim=2).contiguous()
-    mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=DEV)).expand(B, T, T)
-    o_ref, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qkv, mask, False)
+    o_ref, _ = mt.t_scaled_dot_prod_attn_fwd3_t(qkv, None, False)
     assert torch.equal(o, o_ref)
     assert torch.equal(out.view(B, T, H, 64).permute(0, 2, 1, 3), o_ref)
 

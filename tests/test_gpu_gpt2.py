@@ -23,7 +23,7 @@ def to64(params, dtype):
     return [[p.to(dtype).to(torch.float64) for p in grp] for grp in params]
 
 
-def run_case(lo, V, D, L, H, F, T, B, dtype, train, seed=0, pad=True):
+def run_case(lo, V, D, L, H, F, T, B, dtype, train, seed=0, pad=True, mask_as="tensor"):
     params = ogpt2.init_transformer_gpt2(V, D, L, H, F, T, seed=seed)
     g = torch.Generator().manual_seed(seed + 1)
     # make biases / layernorm parameters non-trivial so their gradients are exercised
@@ -36,16 +36,18 @@ def run_case(lo, V, D, L, H, F, T, B, dtype, train, seed=0, pad=True):
         y[0, -5:] = 0                                    # padded tail: labels ignored by the loss
     mask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(B, T, T).contiguous()
     seeds = [1000 + 17 * i for i in range(1 + 3 * L)]
-    grads, (loss, acc, frac) = lo.t_loss_bkwd3_t(to_dev(params, dtype), y.to(DEV), mask.to(DEV), None, train, seeds)
+    dmask = mask.to(DEV) if mask_as == "tensor" else None         # None: the index-masked causal path
+    grads, (loss, acc, frac) = lo.t_loss_bkwd3_t(to_dev(params, dtype), y.to(DEV), dmask, None, train, seeds)
     want_g, (wl, wacc, wfrac) = ogpt2.grad_loss(to64(params, dtype), y, mask, train, seeds)
     return grads, loss, acc, frac, want_g, wl, wacc, wfrac
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("train", [False, True])
-def test_small_model_grads(lo, dtype, train):
+@pytest.mark.parametrize("mask_as", ["tensor", "none"])
+def test_small_model_grads(lo, dtype, train, mask_as):
     grads, loss, acc, frac, want_g, wl, wacc, wfrac = run_case(lo, V=331, D=128, L=2, H=2, F=256, T=128, B=2,
-                                                               dtype=dtype, train=train)
+                                                               dtype=dtype, train=train, mask_as=mask_as)
     ltol, gtol = (1e-5, 5e-5) if dtype == torch.float32 else (5e-3, 2e-2)
     assert abs(loss.item() - wl.item()) <= ltol * abs(wl.item()), (loss.item(), wl.item())
     assert abs(frac.item() - wfrac.item()) < 1e-6
@@ -64,7 +66,8 @@ def test_small_model_grads(lo, dtype, train):
 def test_gpt2_small_config1_fp32(lo):
     # BASELINE config 1: full GPT-2 small, fp32, B=2, T=256, dropout off (eval semantics, x0.9)
     grads, loss, acc, frac, want_g, wl, wacc, wfrac = run_case(lo, V=50257, D=768, L=12, H=12, F=3072, T=256, B=2,
-                                                               dtype=torch.float32, train=False, seed=1234, pad=False)
+                                                               dtype=torch.float32, train=False, seed=1234, pad=False,
+                                                               mask_as="none")
     assert abs(loss.item() - wl.item()) <= 1e-5 * abs(wl.item()), (loss.item(), wl.item())
     worst = 0.0
     for gi, (gg, wg) in enumerate(zip(grads, want_g)):
@@ -89,7 +92,7 @@ def test_loss_curve_short_run(lo, dtype):
     mask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(B, T, T).contiguous()
     master = [[p.clone().to(DEV) for p in grp] for grp in params]
     shadow = None if dtype == torch.float32 else to_dev(params, dtype)
-    moments = lo.init_adam_w(master)
+    _, moments = lo.init_adam_w(master)
     o_params = [[p.double() for p in grp] for grp in params]
     o_mom = [[[torch.zeros_like(p) for p in grp] for grp in o_params] for _ in range(2)]
     got, want = [], []

@@ -19,7 +19,7 @@ def test_adamw_matches_oracle(lo, gdtype):
     wd_mask = [[True, False], [False, True]]
     master = [[p.clone().to(DEV) for p in grp] for grp in params]
     shadow = [[p.to(torch.bfloat16).to(DEV) for p in grp] for grp in params]
-    moments = lo.init_adam_w(master)
+    _, moments = lo.init_adam_w(master)
     o_params = [[p.double() for p in grp] for grp in params]
     o_mom = [[[torch.zeros_like(p) for p in grp] for grp in o_params] for _ in range(2)]
     for i in range(4):
@@ -60,7 +60,7 @@ def test_adamw_multi_equals_single_tensor_calls(lo, pkg):
     wd_mask = [[i % 2 == 0 for i in range(len(sizes))]]
     a_p = [[p.clone().to(DEV) for p in params[0]]]
     a_sh = [[p.to(torch.bfloat16).to(DEV) for p in params[0]]]
-    a_mom = lo.init_adam_w(a_p)
+    _, a_mom = lo.init_adam_w(a_p)
     b_p = [p.clone().to(DEV) for p in params[0]]
     b_sh = [p.to(torch.bfloat16).to(DEV) for p in params[0]]
     b_m = [torch.zeros_like(p) for p in b_p]
