@@ -89,6 +89,21 @@ size_t ptj_colsum_workspace_bytes(int64_t rows, int64_t cols);
 int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes,
                int64_t rows, int64_t cols, int64_t x_row_stride, int dtype, void* stream);
 
+/* ptj_colsum without a workspace argument, for callers that cannot allocate one (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The stage-1 partial sums go to a device array built into
+ * the library (PTJ_COLSUM_STATIC_SCRATCH_BYTES per GPU, held until the process ends); shapes
+ * whose partial sums do not fit -- ptj_colsum_workspace_bytes(rows, cols) above that size --
+ * are rejected with PTJ_ERR_INVALID and nothing is launched.  No hipMalloc, hipFree or other
+ * allocating call is made.  The GPU that `stream` belongs to must be the current device.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls ordered on one stream are safe.  Results are bit-equal
+ * to ptj_colsum's. */
+#define PTJ_COLSUM_STATIC_SCRATCH_BYTES (16u << 20)
+#define PTJ_MAX_DEVICES 64
+int ptj_colsum_static(const void* x, void* out, int64_t rows, int64_t cols, int64_t x_row_stride,
+                      int dtype, void* stream);
+
 /* tanh-GELU forward / backward on a flat array of n elements.
  * Replace t_gelu_fwd_k/_t (model_triton.py:237-260) and t_gelu_bkwd2_k/_t (:274-304). */
 int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);

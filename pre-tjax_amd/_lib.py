@@ -28,6 +28,7 @@ SIGNATURES = {
                                          _int, _p]),
     "ptj_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_colsum": (_int, [_p, _p, _p, _sz, _i64, _i64, _i64, _int, _p]),
+    "ptj_colsum_static": (_int, [_p, _p, _i64, _i64, _i64, _int, _p]),
     "ptj_gelu_fwd": (_int, [_p, _p, _i64, _int, _p]),
     "ptj_gelu_bwd": (_int, [_p, _p, _p, _i64, _int, _p]),
     "ptj_gelu_bwd_colsum": (_int, [_p, _p, _p, _p, _p, _sz, _i64, _i64, _int, _p]),

@@ -5,6 +5,8 @@
 // when shapes allow (VEC = 16/sizeof(T)), scalar otherwise.
 #include "common.h"
 
+#include <mutex>
+
 namespace {
 
 // ---------------------------------------------------------------------------------
@@ -1114,6 +1116,32 @@ int dropout_impl(const void* x, const void* res, void* y, int64_t rows, int64_t 
 
 }  // namespace
 
+// ---- ptj_colsum without a caller workspace ---------------------------------------------
+// The stage-1 partial sums live in a file-scope device array instead of a buffer the caller
+// brings.  Every GPU holds its own copy of the array at its own address, so the address is
+// looked up once per device (with that device current) and kept; kernels receive that
+// pointer, never the array's name, which in host code is only a stand-in.
+static __device__ __align__(256) unsigned char scratch[PTJ_COLSUM_STATIC_SCRATCH_BYTES];
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[PTJ_MAX_DEVICES] = {};
+
+static int colsum_static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return ptj_set_error(PTJ_ERR_LAUNCH, "colsum_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= PTJ_MAX_DEVICES) return ptj_set_error(PTJ_ERR_INVALID, "colsum_static: device index %d", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return ptj_set_error(PTJ_ERR_LAUNCH, "colsum_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PTJ_OK;
+}
+
 extern "C" {
 
 int ptj_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, int64_t rows, int64_t cols,
@@ -1195,6 +1223,25 @@ int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes
     hipStream_t st = (hipStream_t)stream;
     DTYPE_SWITCH(dtype, (colsum_impl<float>(x, out, workspace, workspace_bytes, rows, cols, xs, st)),
                  (colsum_impl<bf16>(x, out, workspace, workspace_bytes, rows, cols, xs, st)));
+}
+
+int ptj_colsum_static(const void* x, void* out, int64_t rows, int64_t cols, int64_t xs, int dtype, void* stream) {
+    PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 31), "colsum_static: bad shape");
+    PTJ_CHECK_ARG(x && out, "colsum_static: null pointer");
+    PTJ_CHECK_ARG(xs >= cols, "colsum_static: row stride smaller than cols");
+    const size_t need = ptj_colsum_workspace_bytes(rows, cols);
+    PTJ_CHECK_ARG(need <= (size_t)PTJ_COLSUM_STATIC_SCRATCH_BYTES,
+                  "colsum_static: [%lld, %lld] needs %zu bytes of partial sums, the built-in scratch holds %zu; "
+                  "use ptj_colsum with a workspace", (long long)rows, (long long)cols, need,
+                  (size_t)PTJ_COLSUM_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    const int rc = colsum_static_scratch(&ws);
+    if (rc != PTJ_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    // every partial that stage 2 reads is written by stage 1 of the same call: nothing in the
+    // scratch needs clearing between calls
+    DTYPE_SWITCH(dtype, (colsum_impl<float>(x, out, ws, need, rows, cols, xs, st)),
+                 (colsum_impl<bf16>(x, out, ws, need, rows, cols, xs, st)));
 }
 
 int ptj_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream) {
