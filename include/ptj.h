@@ -190,6 +190,20 @@ int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64
                    int64_t rows, int64_t cols, int64_t logits_row_stride, int64_t dlogits_row_stride,
                    int dtype, void* stream);
 
+/* ptj_ce_fwd_bwd that also returns the column sums of the stored gradient,
+ * colsum[c] = sum_r dlogits[r, c] -- the `.sum(dim=0)` bias gradient of t_linear_bkwd2_p
+ * (model_triton.py:426) for the layer that produced the logits (the tied LM head,
+ * model_triton.py:2538) -- from the same pass, so the gradient is not read again.
+ * 2-byte storage only (dtype PTJ_BF16); both row strides must be multiples of 8 elements
+ * (all rows then share one 16-byte phase); cols + 8 <= 57344.  Other layouts: call
+ * ptj_ce_fwd_bwd and ptj_colsum.  `workspace`: ptj_ce_colsum_workspace_bytes(rows, cols)
+ * bytes (per-row losses and one fp32 partial row per workgroup).  Fixed summation order. */
+size_t ptj_ce_colsum_workspace_bytes(int64_t rows, int64_t cols);
+int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss, int64_t* count,
+                          void* dlogits, int64_t* pred, void* colsum, void* workspace,
+                          size_t workspace_bytes, int64_t rows, int64_t cols, int64_t logits_row_stride,
+                          int64_t dlogits_row_stride, int dtype, void* stream);
+
 /* ---- dense contraction --------------------------------------------------- */
 
 /* C[n,m] = sum_k A(n,k) * B(k,m) (+ bias[m]) (gelu) with fp32 accumulation on MFMA.

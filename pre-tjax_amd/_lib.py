@@ -42,6 +42,8 @@ SIGNATURES = {
     "ptj_log_softmax_bwd": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_ce_workspace_bytes": (_sz, [_i64]),
     "ptj_ce_fwd_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
+    "ptj_ce_colsum_workspace_bytes": (_sz, [_i64, _i64]),
+    "ptj_ce_fwd_bwd_colsum": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "ptj_gemm": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p, _i64, _p, _sz, _int,
                         _p]),

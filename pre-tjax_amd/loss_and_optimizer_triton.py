@@ -10,15 +10,19 @@ from .model_triton import _workspace
 from .spec_torch import accuracy, t_avg_cross_entropy_loss, t_avg_cross_entropy_loss_bkwd3  # noqa: F401  (torch twins)
 
 
-def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Tensor, inplace=False, want_pred=False):
+def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Tensor, inplace=False, want_pred=False,
+                                     want_colsum=False):
     """Fused log-softmax + mean cross-entropy forward and backward
     (reference: loss_and_optimizer_triton.py:176-197).
 
     Returns ``(loss[1] fp32, nonzero_count 0-d int64, dloss_dlogits like x_logits)``.
     With ``inplace=True`` the gradient overwrites ``x_logits`` (an extension: the
-    reference always allocates).  With ``want_pred=True`` a fourth value is returned:
+    reference always allocates).  With ``want_pred=True`` a further value is returned:
     the row-wise argmax of the logits (int64, shaped like ``y_labels``), computed in
-    the same pass -- the input of ``accuracy``."""
+    the same pass -- the input of ``accuracy``.  With ``want_colsum=True`` the last value
+    returned is the column sum of the stored gradient over all rows (``[V]``: the gradient
+    of the bias that was added to the logits, model_triton.py:426), from the same pass for
+    2-byte logits whose row pitch is a multiple of 8 elements, else from ``colsum_t``."""
     require_gpu(y_labels, x_logits)
     shape = x_logits.shape
     labels = y_labels.reshape(-1).to(torch.int64).contiguous()
@@ -33,14 +37,31 @@ def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Ten
     else:  # same row pitch as the logits, so rows keep their 16-byte phase
         dx = torch.empty_strided((rows, cols), (x2.stride(0), 1), dtype=x2.dtype, device=x2.device)
     pred = torch.empty(rows, dtype=torch.int64, device=x2.device) if want_pred else None
-    ws_bytes = lib().ptj_ce_workspace_bytes(rows)
-    ws = _workspace(ws_bytes, x2.device, "ce")
-    check(lib().ptj_ce_fwd_bwd(ptr(labels), ptr(x2), ptr(loss), ptr(count), ptr(dx), ptr(pred), ptr(ws), ws_bytes, rows, cols,
-                               x2.stride(0), dx.stride(0), dtype_code(x2), stream()), "ptj_ce_fwd_bwd")
+    colsum = None
+    fused = (want_colsum and x2.dtype == torch.bfloat16 and x2.stride(0) % 8 == 0 and dx.stride(0) % 8 == 0
+             and cols + 8 <= 1024 * 56 and (x2.data_ptr() - dx.data_ptr()) % 16 == 0)
+    if fused:
+        colsum = torch.empty(cols, dtype=x2.dtype, device=x2.device)
+        ws_bytes = lib().ptj_ce_colsum_workspace_bytes(rows, cols)
+        ws = _workspace(ws_bytes, x2.device, "ce")
+        check(lib().ptj_ce_fwd_bwd_colsum(ptr(labels), ptr(x2), ptr(loss), ptr(count), ptr(dx), ptr(pred), ptr(colsum),
+                                          ptr(ws), ws_bytes, rows, cols, x2.stride(0), dx.stride(0), dtype_code(x2),
+                                          stream()), "ptj_ce_fwd_bwd_colsum")
+    else:
+        ws_bytes = lib().ptj_ce_workspace_bytes(rows)
+        ws = _workspace(ws_bytes, x2.device, "ce")
+        check(lib().ptj_ce_fwd_bwd(ptr(labels), ptr(x2), ptr(loss), ptr(count), ptr(dx), ptr(pred), ptr(ws), ws_bytes, rows,
+                                   cols, x2.stride(0), dx.stride(0), dtype_code(x2), stream()), "ptj_ce_fwd_bwd")
+        if want_colsum:
+            from .model_triton import colsum_t
+            colsum = colsum_t(dx)
     dx = dx.view(shape) if inplace else dx.reshape(shape)
+    out = (loss, count, dx)
     if want_pred:
-        return loss, count, dx, pred.reshape(y_labels.shape)
-    return loss, count, dx
+        out += (pred.reshape(y_labels.shape),)
+    if want_colsum:
+        out += (colsum,)
+    return out
 
 
 def accuracy_from_pred(y_labels, pred):
@@ -56,9 +77,10 @@ def t_loss_bkwd3_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
     y_in = y[:, :-1]
     y_out = y[:, 1:]
     logits, acts = t_gpt2_forward_with_acts_t(params, y_in, y_mask, y_indices, train, p_gen_aux)
-    loss_val, tokens_count, dloss_dx, pred = t_avg_cross_entropy_loss_bkwd3_t(y_out, logits, inplace=True,
-                                                                             want_pred=True)
-    grads = t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y_in, y_mask, y_indices, train, p_gen_aux)
+    # the bias gradient of the tied head (column sums of the loss gradient) comes out of the loss pass
+    loss_val, tokens_count, dloss_dx, pred, dbemb = t_avg_cross_entropy_loss_bkwd3_t(y_out, logits, inplace=True,
+                                                                                    want_pred=True, want_colsum=True)
+    grads = t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y_in, y_mask, y_indices, train, p_gen_aux, dbemb=dbemb)
     acc = accuracy_from_pred(y_out, pred)
     return grads, (loss_val, acc, tokens_count / y_out.numel())
 

@@ -655,8 +655,9 @@ def t_gpt2_forward_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
     return t_gpt2_forward_with_acts_t(params, y, y_mask, y_indices, train, p_gen_aux)[0]
 
 
-def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_aux=None):
-    """model_triton.py:2583-2593 + :2489-2521: gradient nest shaped like `params`."""
+def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_aux=None, *, dbemb=None):
+    """model_triton.py:2583-2593 + :2489-2521: gradient nest shaped like `params`.
+    `dbemb`, if given, is colsum_t(dloss_dx) already computed by the producer of dloss_dx."""
     L = len(params) - 3
     if not train:
         p_gen_aux = [0] * (1 + 3 * L)
@@ -669,7 +670,8 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
     if dlog.stride(1) != 1:
         dlog = dlog.contiguous()
     h2d = h.view(N, D)
-    dbemb = colsum_t(dlog)
+    if dbemb is None:
+        dbemb = colsum_t(dlog)
     dwemb = matmul_t(dlog.t(), h2d)                                     # [V,D]  LM-head weight grad
     dh = matmul_t(dlog, wemb)                                           # [N,D]
     # Every dropout backward acts on a gradient that a LayerNorm backward has just produced,

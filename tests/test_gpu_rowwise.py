@@ -167,6 +167,36 @@ def test_ce_fwd_bwd(lo, dtype, rows, V):
     assert dx3.data_ptr() == xin.data_ptr() and torch.equal(dx3, dx) and torch.equal(loss3, loss)
 
 
+@pytest.mark.parametrize("rows,V,pitch", [(512, 50257, 50304), (300, 1000, 1000), (64, 35374, 35376), (5, 17, 24),
+                                          (1030, 4099, 4104)])
+def test_ce_with_column_sums_equals_separate_passes(lo, mt, rows, V, pitch):
+    """The loss pass that also sums the gradient's columns (2-byte logits, row pitch a multiple
+    of 8): loss, count, gradient and argmax bit-equal to the plain pass, and the sums equal to
+    the fp64 column sums of the stored gradient within the rounding of the 2-byte result."""
+    g = gen(66)
+    buf = randn(g, rows, pitch, dtype=torch.bfloat16).to(DEV)
+    x = buf[:, :V]
+    y = torch.randint(0, V, (rows,), generator=g)
+    y[::5] = 0
+    y = y.to(DEV)
+    loss0, cnt0, dx0, pred0 = lo.t_avg_cross_entropy_loss_bkwd3_t(y, x, want_pred=True)
+    loss1, cnt1, dx1, pred1, sums = lo.t_avg_cross_entropy_loss_bkwd3_t(y, x, want_pred=True, want_colsum=True)
+    assert torch.equal(loss0, loss1) and torch.equal(cnt0, cnt1) and torch.equal(pred0, pred1)
+    assert torch.equal(dx0, dx1)
+    want = f64(dx1).sum(0)
+    assert sums.shape == (V,) and sums.dtype == torch.bfloat16
+    err = (f64(sums) - want).abs()
+    assert (err <= 2 ** -8 * want.abs() + 1e-9).all(), err.max().item()
+    # against the two-pass form the fused call replaces (fp32 partial sums in another order)
+    ref = mt.colsum_t(dx0)
+    assert (f64(sums) - f64(ref)).abs().max().item() <= 2 ** -7 * want.abs().max().item() + 1e-9
+    # in place, as the training step calls it; a second call gives the same bits
+    xin = buf.clone()[:, :V]
+    loss2, _, dx2, _, sums2 = lo.t_avg_cross_entropy_loss_bkwd3_t(y, xin, inplace=True, want_pred=True, want_colsum=True)
+    assert dx2.data_ptr() == xin.data_ptr() and torch.equal(dx2, dx0) and torch.equal(sums2, sums)
+    assert torch.equal(loss2, loss0)
+
+
 def test_ce_all_labels_zero_is_nan(lo):
     x = torch.randn(4, 50, device=DEV)
     loss, cnt, dx = lo.t_avg_cross_entropy_loss_bkwd3_t(torch.zeros(4, dtype=torch.int64, device=DEV), x)
