@@ -19,14 +19,24 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# Measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this benchmark (commands, per-kernel table
-# and the copy-kernel scale factors: profiles/hbm_traffic__gpt2_b16_t1024_bf16_step.md): 228.3e6 read +
-# 69.3e6 written per GEMM launch, averaged over the forward, dX and dW products of a step.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 237.9e6
+# HBM bytes per GEMM launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark: read from
+# the data file that is written together with the profiles/ summary of those runs (commands, per-kernel table
+# and copy-kernel scale factors are in that summary); null when the file is missing.
+GEMM_TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_traffic__gpt2_b16_t1024_bf16_step.json")
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 matrix
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 CFG = dict(V=50257, D=768, L=12, H=12, F=3072, T=1024, B=16)
+
+
+def gemm_traffic():
+    try:
+        with open(GEMM_TRAFFIC_FILE) as f:
+            d = json.load(f)
+        return float(d["fetch_bytes_per_launch"]) + float(d["write_bytes_per_launch"]), d
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def step_flops(c):
@@ -62,12 +72,164 @@ def make_state(torch, lo, c, dev):
     return master, shadow, moments, wd_mask
 
 
+def _timeit(torch, fn, n=20, warm=3):
+    for _ in range(warm):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(n):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / n
+
+
+def _timeit_sets(torch, fn, nsets, n=24):
+    """fn(i) works on buffer set i; the sets together exceed the 256 MB last-level cache, so the
+    rates are HBM rates as in the training step (a leg that re-used one set would run out of cache)."""
+    for i in range(3):
+        fn(i % nsets)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for i in range(n):
+        fn(i % nsets)
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / n
+
+
+def attn_leg(torch, mt, B, H, T, dh, dtype, train, mask_tensor=False):
+    dev = "cuda:0"
+    qkv = torch.randn(B, H, 3, T, dh, device=dev).to(dtype)
+    dO = torch.randn(B, H, T, dh, device=dev).to(dtype)
+    q, k, v = qkv.unbind(2)
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=dev)).expand(B, T, T).contiguous() if mask_tensor else None
+    o, ms_, ls_ = mt.attn_fwd_t(q, k, v, mask, train, 5)
+    t_af = _timeit(torch, lambda: mt.attn_fwd_t(q, k, v, mask, train, 5))
+    t_ab = _timeit(torch, lambda: mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, mask, train, 5))
+    causal = dh * B * H * T * (T + 1) // 2
+    peak = PEAK_BF16_TFLOPS if dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
+    tot = 14 * causal / ((t_af + t_ab) * 1e-3) / 1e12
+    return {"fwd_ms": round(t_af, 4), "bwd_ms": round(t_ab, 4),
+            "fwd_tflops": round(4 * causal / (t_af * 1e-3) / 1e12, 1),
+            "bwd_tflops": round(10 * causal / (t_ab * 1e-3) / 1e12, 1),
+            "fwd_bwd_tflops": round(tot, 1), "peak_tflops": peak, "frac": round(tot / peak, 4)}
+
+
+def rowwise_leg(torch, mt, lo, N, D, F, V):
+    """Row-wise kernels at the training step's shapes, bf16, algorithmic bytes / HBM peak."""
+    dev = "cuda:0"
+    ND, NF = 12, 4                                   # 12 x 3 x 25 MB and 4 x 2 x 100 MB
+    bf = torch.bfloat16
+    xs_ = [torch.randn(N, D, device=dev).to(bf) for _ in range(ND)]
+    dys = [torch.randn(N, D, device=dev).to(bf) for _ in range(ND)]
+    rss = [torch.randn(N, D, device=dev).to(bf) for _ in range(ND)]
+    gam = torch.ones(D, device=dev, dtype=bf)
+    xfs = [torch.randn(N, F, device=dev).to(bf) for _ in range(NF)]
+    dfs = [torch.randn(N, F, device=dev).to(bf) for _ in range(NF)]
+    keeps = [mt.dropout_add_t(xs_[i], rss[i], True, 42, want_keep=True)[1] for i in range(ND)]
+    e2 = 2
+    rows = {}
+
+    def gbs(nbytes, ms):
+        return round(nbytes / (ms * 1e-3) / 1e9, 1)
+    ts = lambda fn, n: _timeit_sets(torch, fn, n)
+    rows["layernorm_fwd"] = gbs(2 * N * D * e2, ts(lambda i: mt.t_layernorm_fwd_t((gam, gam), xs_[i]), ND))
+    rows["layernorm_bwd_dx_dgb"] = gbs(3 * N * D * e2, ts(lambda i: mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i]), ND))
+    # the training step's variants: residual update + norm in one pass (reads x, res; writes y, h,
+    # keep bytes), and the norm backward that adds the residual and also writes the dropped copy
+    # and its column sums (reads dy, x, res, keep bytes; writes dx, dropped)
+    rows["dropout_add_layernorm"] = gbs(4 * N * D * e2 + N * D // 8, ts(
+        lambda i: mt.dropout_add_layernorm_t(xs_[i], rss[i], (gam, gam), True, 42, want_keep=True), ND))
+    rows["layernorm_bwd_res_drop_sums"] = gbs(5 * N * D * e2 + N * D // 8, ts(
+        lambda i: mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i], residual=rss[i], drop=(True, 42, keeps[i]),
+                                       drop_sum=True), ND))
+    rows["gelu_fwd"] = gbs(2 * N * F * e2, ts(lambda i: mt.t_gelu_fwd_t(xfs[i]), NF))
+    rows["gelu_bwd"] = gbs(3 * N * F * e2, ts(lambda i: mt.t_gelu_bkwd2_t(dfs[i], xfs[i]), NF))
+    rows["gelu_bwd_colsum"] = gbs(3 * N * F * e2, ts(lambda i: mt.t_gelu_bkwd2_colsum_t(dfs[i], xfs[i]), NF))
+    rows["dropout_fwd"] = gbs(2 * N * D * e2, ts(lambda i: mt.t_dropout_fwd_t(xs_[i], True, 42), ND))
+    # a plain device copy of the same size as the LayerNorm legs (25 MB read + 25 MB written), for scale
+    cps = [torch.empty_like(xs_[0]) for _ in range(ND)]
+    rows["copy_25MB_for_scale"] = gbs(2 * N * D * e2, ts(lambda i: cps[i].copy_(xs_[i]), ND))
+    del xfs, dfs
+    # the logits as the step holds them: rows padded to a multiple of 64 columns (the LM-head product's
+    # output pitch), argmax and the column sums of the gradient requested, as the step does; the gradient
+    # goes to a second buffer here (in place the next timed call would read gradients as logits)
+    vp = (V + 63) // 64 * 64
+    lgbuf = torch.randn(N, vp, device=dev).to(bf)
+    lg = lgbuf[:, :V]
+    lab = torch.randint(0, V, (N,), device=dev)
+    rows["ce_fwd_bwd"] = gbs(2 * N * V * e2 + 8 * N, _timeit(
+        torch, lambda: lo.t_avg_cross_entropy_loss_bkwd3_t(lab, lg, want_pred=True), n=8))
+    rows["ce_fwd_bwd_colsum"] = gbs(2 * N * V * e2 + 8 * N, _timeit(
+        torch, lambda: lo.t_avg_cross_entropy_loss_bkwd3_t(lab, lg, want_pred=True, want_colsum=True), n=8))
+    del lg, lgbuf
+    return {"achieved_GBs": rows, "peak_GBs": PEAK_HBM_GBS, "bytes": "algorithmic (minimum traffic), bf16",
+            "note": "wrapper calls timed with HIP events (two launches each where a second-stage reduction "
+                    "follows); inputs rotate over buffer sets larger than the last-level cache; "
+                    "dropout_fwd and dropout_add_layernorm evaluate one Philox4x32-10 per element (20 "
+                    "quarter-rate 32x32->64-bit multiplies), which bounds them below the HBM rate",
+            "frac": {kk: round(vv / PEAK_HBM_GBS, 3) for kk, vv in rows.items()}}
+
+
+def c3_leg(torch, mt, dtype):
+    """BASELINE configuration 3: row-wise kernels on N = 8192 rows.  Each entry is
+    [GB/s by algorithmic bytes, GB/s by the reference's 3 * numel * element_size convention]."""
+    dev = "cuda:0"
+    N, D, F = 8192, 768, 3072
+    e = 2 if dtype == torch.bfloat16 else 4
+    NS = 16 if e == 2 else 8
+    g = torch.Generator(device="cpu").manual_seed(1234 + 2)
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(dtype).to(dev)
+    xs_, dys = [mk(N, D) for _ in range(NS)], [mk(N, D) for _ in range(NS)]
+    gam, bet = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype).to(dev), (0.1 * torch.randn(D, generator=g)).to(dtype).to(dev)
+    xf, df = [mk(N, F) for _ in range(4)], [mk(N, F) for _ in range(4)]
+    out = {}
+
+    def both(alg_streams, numel, ms):
+        return [round(alg_streams * numel * e / (ms * 1e-3) / 1e9, 1), round(3 * numel * e / (ms * 1e-3) / 1e9, 1)]
+    ts = lambda fn, n: _timeit_sets(torch, fn, n)
+    out["layernorm_fwd"] = both(2, N * D, ts(lambda i: mt.t_layernorm_fwd_t((gam, bet), xs_[i]), NS))
+    out["layernorm_bwd_x"] = both(3, N * D, ts(lambda i: mt.t_layernorm_bkwd2_x_t(dys[i], (gam, bet), xs_[i]), NS))
+    out["layernorm_bwd_p"] = both(2, N * D, ts(lambda i: mt.t_layernorm_bkwd2_p_t(dys[i], (gam, bet), xs_[i]), NS))
+    out["layernorm_bwd_x_and_p_one_pass"] = both(3, N * D, ts(lambda i: mt.layernorm_bkwd2_t(dys[i], (gam, bet), xs_[i]), NS))
+    out["gelu_fwd"] = both(2, N * F, ts(lambda i: mt.t_gelu_fwd_t(xf[i]), 4))
+    out["gelu_bwd"] = both(3, N * F, ts(lambda i: mt.t_gelu_bkwd2_t(df[i], xf[i]), 4))
+    out["dropout_fwd"] = both(2, N * D, ts(lambda i: mt.t_dropout_fwd_t(xs_[i], True, 42), NS))
+    out["dropout_bwd"] = both(2, N * D, ts(lambda i: mt.t_dropout_bkwd2_t(dys[i], xs_[i], True, 42), NS))
+    return out
+
+
+def c4_leg(torch, mt, lo, dtype):
+    """BASELINE configuration 4: LM head x[8192,768] . W[50257,768]^T then fused log-softmax +
+    mean cross-entropy forward and backward."""
+    dev = "cuda:0"
+    N, D, V = 8192, 768, 50257
+    e = 2 if dtype == torch.bfloat16 else 4
+    g = torch.Generator(device="cpu").manual_seed(1234 + 3)
+    x = torch.randn(N, D, generator=g).to(dtype).to(dev)
+    w = (0.02 * torch.randn(V, D, generator=g)).to(dtype).to(dev)
+    b = torch.zeros(V, dtype=dtype, device=dev)
+    lab = torch.randint(0, V, (N,), generator=g).to(dev)
+    logits = mt._padded_logits(N, V, dtype, dev)
+    t_mm = _timeit(torch, lambda: mt.matmul_t(x, w.t(), b, out=logits), n=8)
+    dl = torch.empty_strided(logits.shape, logits.stride(), dtype=dtype, device=dev)
+    mt.matmul_t(x, w.t(), b, out=logits)
+    t_ce = _timeit(torch, lambda: lo.t_avg_cross_entropy_loss_bkwd3_t(lab, logits), n=8)
+    peak = PEAK_BF16_TFLOPS if dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
+    tf = 2.0 * N * D * V / (t_mm * 1e-3) / 1e12
+    return {"gemm_ms": round(t_mm, 3), "gemm_tflops": round(tf, 1), "gemm_frac_of_mfma_peak": round(tf / peak, 4),
+            "ce_ms": round(t_ce, 3), "ce_GBs_algorithmic": round((2 * N * V * e + 8 * N) / (t_ce * 1e-3) / 1e9, 1),
+            "ce_GBs_3numel": round(3 * N * V * e / (t_ce * 1e-3) / 1e9, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the legs of baseline configurations 2, 3 and 4")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run one plain 1 GiB device copy first (reference reading for FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--steps-only", action="store_true",
@@ -149,107 +311,50 @@ def main():
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
 
     # ---- attention and row-wise kernels at the workload's shapes (HIP events) ----------------
-    def timeit(fn, n=20):
-        for _ in range(3):
-            fn()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(n):
-            fn()
-        e.record()
-        torch.cuda.synchronize()
-        return s.elapsed_time(e) / n
-
     H, dh, D, F = c["H"], c["D"] // c["H"], c["D"], c["F"]
     N = B * T
-    qkv = torch.randn(B, H, 3, T, dh, device=dev).to(torch.bfloat16)
-    dO = torch.randn(B, H, T, dh, device=dev).to(torch.bfloat16)
-    q, k, v = qkv.unbind(2)
-    o, ms_, ls_ = mt.attn_fwd_t(q, k, v, None, True, 5)
-    t_af = timeit(lambda: mt.attn_fwd_t(q, k, v, None, True, 5))
-    t_ab = timeit(lambda: mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, None, True, 5))
-    causal = dh * B * H * T * (T + 1) // 2
-    attn = {"fwd_ms": round(t_af, 4), "bwd_ms": round(t_ab, 4),
-            "fwd_tflops": round(4 * causal / (t_af * 1e-3) / 1e12, 1),
-            "bwd_tflops": round(10 * causal / (t_ab * 1e-3) / 1e12, 1),
-            "fwd_bwd_tflops": round(14 * causal / ((t_af + t_ab) * 1e-3) / 1e12, 1),
-            "peak_tflops": PEAK_BF16_TFLOPS,
-            "frac": round(14 * causal / ((t_af + t_ab) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-            "shape": "B%d H%d T%d dh%d bf16 causal dropout0.1" % (B, H, T, dh)}
-    # Row-wise legs: every call works on another set of buffers and the sets together exceed the
-    # 256 MB last-level cache, so the rates are HBM rates as in the training step (a leg that
-    # re-used one set would run out of cache).
-    def timeit_sets(fn, nsets, n=24):
-        for i in range(3):
-            fn(i % nsets)
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for i in range(n):
-            fn(i % nsets)
-        e.record()
-        torch.cuda.synchronize()
-        return s.elapsed_time(e) / n
+    attn = attn_leg(torch, mt, B, H, T, dh, torch.bfloat16, train=True)
+    attn["shape"] = "B%d H%d T%d dh%d bf16 causal dropout0.1" % (B, H, T, dh)
+    rowwise = rowwise_leg(torch, mt, lo, N, D, F, V)
 
-    ND, NF = 12, 4                                   # 12 x 3 x 25 MB and 4 x 2 x 100 MB
-    xs_ = [torch.randn(N, D, device=dev).to(torch.bfloat16) for _ in range(ND)]
-    dys = [torch.randn(N, D, device=dev).to(torch.bfloat16) for _ in range(ND)]
-    rss = [torch.randn(N, D, device=dev).to(torch.bfloat16) for _ in range(ND)]
-    gam = torch.ones(D, device=dev, dtype=torch.bfloat16)
-    xfs = [torch.randn(N, F, device=dev).to(torch.bfloat16) for _ in range(NF)]
-    dfs = [torch.randn(N, F, device=dev).to(torch.bfloat16) for _ in range(NF)]
-    keeps = [mt.dropout_add_t(xs_[i], rss[i], True, 42, want_keep=True)[1] for i in range(ND)]
-    e2 = 2
-    rows = {}
-
-    def gbs(nbytes, ms):
-        return round(nbytes / (ms * 1e-3) / 1e9, 1)
-    rows["layernorm_fwd"] = gbs(2 * N * D * e2, timeit_sets(lambda i: mt.t_layernorm_fwd_t((gam, gam), xs_[i]), ND))
-    rows["layernorm_bwd_dx_dgb"] = gbs(3 * N * D * e2,
-                                       timeit_sets(lambda i: mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i]), ND))
-    # the training step's variants: residual update + norm in one pass (reads x, res; writes y, h,
-    # keep bytes), and the norm backward that adds the residual and also writes the dropped copy
-    # and its column sums (reads dy, x, res, keep bytes; writes dx, dropped)
-    rows["dropout_add_layernorm"] = gbs(4 * N * D * e2 + N * D // 8, timeit_sets(
-        lambda i: mt.dropout_add_layernorm_t(xs_[i], rss[i], (gam, gam), True, 42, want_keep=True), ND))
-    rows["layernorm_bwd_res_drop_sums"] = gbs(5 * N * D * e2 + N * D // 8, timeit_sets(
-        lambda i: mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i], residual=rss[i], drop=(True, 42, keeps[i]),
-                                       drop_sum=True), ND))
-    rows["gelu_fwd"] = gbs(2 * N * F * e2, timeit_sets(lambda i: mt.t_gelu_fwd_t(xfs[i]), NF))
-    rows["gelu_bwd"] = gbs(3 * N * F * e2, timeit_sets(lambda i: mt.t_gelu_bkwd2_t(dfs[i], xfs[i]), NF))
-    rows["gelu_bwd_colsum"] = gbs(3 * N * F * e2, timeit_sets(lambda i: mt.t_gelu_bkwd2_colsum_t(dfs[i], xfs[i]), NF))
-    rows["dropout_fwd"] = gbs(2 * N * D * e2, timeit_sets(lambda i: mt.t_dropout_fwd_t(xs_[i], True, 42), ND))
-    del xfs, dfs
-    # the logits as the step holds them: rows padded to a multiple of 64 columns (the LM-head product's
-    # output pitch), argmax requested; the gradient goes to a second buffer here (in place the next timed
-    # call would read gradients as logits)
-    vp = (V + 63) // 64 * 64
-    lgbuf = torch.randn(N, vp, device=dev).to(torch.bfloat16)
-    lg = lgbuf[:, :V]
-    lab = torch.randint(0, V, (N,), device=dev)
-    rows["ce_fwd_bwd"] = gbs(2 * N * V * e2 + 8 * N,
-                             timeit(lambda: lo.t_avg_cross_entropy_loss_bkwd3_t(lab, lg, want_pred=True), n=8))
-    del lg, lgbuf
-    rowwise = {"achieved_GBs": rows, "peak_GBs": PEAK_HBM_GBS, "bytes": "algorithmic (minimum traffic), bf16",
-               "note": "wrapper calls timed with HIP events (two launches each where a second-stage reduction "
-                       "follows); inputs rotate over buffer sets larger than the last-level cache",
-               "frac": {kk: round(vv / PEAK_HBM_GBS, 3) for kk, vv in rows.items()}}
+    # ---- the other configurations of the baseline, as extra legs ---------------------------------
+    extra = None
+    if not args.no_extra:
+        extra = {"C2_attention_B8_H12_T1024_dh64": {
+                     "bf16": attn_leg(torch, mt, 8, 12, 1024, 64, torch.bfloat16, train=False),
+                     "fp32": attn_leg(torch, mt, 8, 12, 1024, 64, torch.float32, train=False),
+                     "bf16_bool_mask_tensor": attn_leg(torch, mt, 8, 12, 1024, 64, torch.bfloat16, train=False,
+                                                       mask_tensor=True),
+                     "note": "causal, eval mode (x0.9), HIP events; flops = (4 | 10) * dh * B * H * T(T+1)/2; "
+                             "bool_mask_tensor: the same lower-triangular mask given as a [B,T,T] bool tensor "
+                             "(bit-packed on the device once per tensor, applied from the packed words)"},
+                 "C3_rowwise_N8192": {"bf16": c3_leg(torch, mt, torch.bfloat16), "fp32": c3_leg(torch, mt, torch.float32),
+                                      "note": "GB/s: algorithmic bytes | the reference's 3*numel*element_size "
+                                              "convention (tests/test_t_speed_t_layernorm_fwd.py:101)"},
+                 "C4_lm_head_ce_N8192": {"bf16": c4_leg(torch, mt, lo, torch.bfloat16),
+                                         "fp32": c4_leg(torch, mt, lo, torch.float32)}}
 
     # ---- CPU baseline: the oracle (fp32) on a bounded sample ------------------------------------
     cpu = None
     if not args.no_cpu:
         from oracle import gpt2 as ogpt2
         nthreads = torch.get_num_threads()
-        cb = 8                                   # about 15 s of CPU work on 16 host cores
+        cb = 2                                   # 2 of the 16 sequences: about 7 s per run on 16 host cores
         cparams = [[p.detach().to("cpu") for p in grp] for grp in master]
         cy = tokens[0, :cb].to("cpu")
         cmask = torch.tril(torch.ones(T, T, dtype=torch.bool)).expand(cb, T, T)
-        t1 = time.perf_counter()
-        ogpt2.grad_loss(cparams, cy, cmask, False)
-        cpu_s = time.perf_counter() - t1
+        runs = []
+        for r in range(4):                       # one warm-up, then three timed runs: the median counts
+            t1 = time.perf_counter()
+            ogpt2.grad_loss(cparams, cy, cmask, True, seeds[0])
+            runs.append(time.perf_counter() - t1)
+        cpu_s = sorted(runs[1:])[1]
         cpu = {"value": round(1.0 / (cpu_s * (B / cb)), 5), "unit": "it/s", "cores": nthreads, "kind": "port",
-               "sample": "oracle fwd+bwd (torch fp32 autograd, eval-mode dropout scaling) on %d of %d sequences, "
-                         "%.2f s, scaled to the full batch" % (cb, B, cpu_s)}
+               "sample": "oracle fwd+bwd (torch fp32 autograd, train mode with the step's Philox seeds) on %d of %d "
+                         "sequences: warm-up + median of 3 runs = %.2f s, scaled to the full batch"
+                         % (cb, B, cpu_s)}
 
+    traffic, traffic_src = gemm_traffic()
     out = {
         "metric": "GPT-2 113M fwd+bwd it/s at B16 T1024; attn fwd+bwd TFLOP/s vs MFMA peak",
         "value": round(value, 4), "unit": "it/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -260,9 +365,10 @@ def main():
                    "global_batch": B, "seq_len": T, "step_tflop": round(total_flops / 1e12, 3),
                    "step_tflops_achieved": round(total_flops / 1e12 * value, 1)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
-                     "traffic_note": "HBM bytes per GEMM launch (average over the 147 launches of a step) from rocprofv3 "
-                                     "FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy; algorithmic minimum 145.2e6",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                     "traffic_note": "bytes per GEMM launch at the L2 boundary (average over the launches of a step) from "
+                                     "rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy, read from "
+                                     "profiles/%s; algorithmic minimum 145.2e6" % os.path.basename(GEMM_TRAFFIC_FILE),
                      "kernel": "gemm_kernel<bf16> (all %d launches of a step: fwd, dX, dW)" % (n_launch // args.steps),
                      "avg_launch_ms": round(gemm_ms / n_launch, 4),
                      "gflop_per_launch": round(gemm_flops / n_launch / 1e9, 2),
@@ -270,6 +376,7 @@ def main():
         "attn": attn,
         "rowwise": rowwise,
         "cpu_baseline": cpu,
+        "extra": extra,
         "final_loss": round(float(losses[-1].item()), 4),
     }
     print(json.dumps(out))

@@ -34,10 +34,42 @@ namespace {
 #define PTJ_GEMM_BM 256
 #endif
 constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from B)
-constexpr int WAVES_N = 2;                  // (BM/64) x 2 wavefronts, each 64 rows x 96 columns
-constexpr int GEMM_THREADS = (BM / 64) * WAVES_N * 64;
-constexpr int TM = 2, TN = 3;           // 32x32 MFMA tiles per wavefront
-constexpr int NUM_CUS = 256;            // persistent grid: one workgroup per CU
+#ifndef PTJ_GEMM_TM
+#define PTJ_GEMM_TM 2
+#endif
+// Register sets that stage operand panels between HBM and LDS: with 2, the loads of panel
+// kt+2 are issued during step kt and have one step to arrive; with 3, panel kt+3 is requested
+// during step kt and has two.
+#ifndef PTJ_GEMM_STAGES
+#define PTJ_GEMM_STAGES 2
+#endif
+constexpr int STAGES = PTJ_GEMM_STAGES;
+static_assert(STAGES == 2 || STAGES == 3, "two or three staging register sets");
+constexpr int TM = PTJ_GEMM_TM, TN = 3;     // 32x32 MFMA tiles per wavefront (rows x columns)
+constexpr int WROWS = TM * 32;              // C rows per wavefront
+constexpr int WAVES_N = 2;                  // (BM/WROWS) x 2 wavefronts, each WROWS rows x 96 columns
+constexpr int GEMM_THREADS = (BM / WROWS) * WAVES_N * 64;
+constexpr int DEFAULT_CUS = 256;        // MI355X; used only when no device can be queried (planning calls without a GPU)
+
+// Compute units of the current device (persistent grid: one workgroup per CU), asked once per
+// device and kept.
+int num_cus() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return DEFAULT_CUS;
+    }
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = DEFAULT_CUS;
+        }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 
 // threadIdx.x behind an opaque barrier: everything derived from it (LDS and global
 // offsets) is recomputed per call instead of being hoisted out of the persistent tile
@@ -114,7 +146,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& g, f32x16 (&acc)[TN][TM
 #define GEMM_READ_CHUNK(C, BUF)                                                                              \
     do {                                                                                                     \
         const int q__ = (C) * 2 + lg;                                                                        \
-        _Pragma("unroll") for (int t = 0; t < TM; ++t) fa[BUF][t] = read_frag<T>(cA, wm * 64 + t * 32 + lr, q__); \
+        _Pragma("unroll") for (int t = 0; t < TM; ++t) fa[BUF][t] = read_frag<T>(cA, wm * WROWS + t * 32 + lr, q__); \
         _Pragma("unroll") for (int t = 0; t < TN; ++t) fb[BUF][t] = read_frag<T>(cB, wn * 96 + t * 32 + lr, q__); \
     } while (0)
         GEMM_READ_CHUNK(0, 0);
@@ -153,7 +185,7 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
                                               int row0, int col0, int kbeg, int nk) {
     constexpr int BK = BKB / (int)sizeof(T);
     constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
-    static_assert(TN == 3 && TM == 2, "the pipeline below is written for 2x3 MFMA tiles per wavefront");
+    static_assert(TN == 3, "the pipeline below is written for three MFMA tile columns per wavefront");
     if (nk <= 0) return;
     const int tid = fresh_tid();
     const int lane = tid & 63, wave = tid >> 6;
@@ -163,11 +195,11 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
     const T* B = (const T*)g.b;
     char* sA = smem;
     char* sB = smem + 2 * A_BYTES;
-    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1;
-    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1;
+    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1, la2;
+    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1, lb2;
     typename Frag<T>::type fa[2][TM], fb[TN], fx[TN];
     const int last = nk - 1;
-    const int arow = wm * 64 + lr, brow = wn * 96 + lr;
+    const int arow = wm * WROWS + lr, brow = wn * 96 + lr;
 
 #define SB() __builtin_amdgcn_sched_barrier(0)
 #define K0_OF(KT) (kbeg + ((KT) < last ? (KT) : last) * BK)
@@ -225,16 +257,34 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
     lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(0), tid, g.m);
     la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(1), tid, g.n);
     lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(1), tid, g.m);
+    if constexpr (STAGES == 3) {
+        la2.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(2), tid, g.n);
+        lb2.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(2), tid, g.m);
+    }
     la0.store(sA, tid);
     lb0.store(sB, tid);
     __syncthreads();
     RD_A(0, 0, 0); RD_B(fb[0], 0, 0, 0); RD_B(fb[1], 0, 0, 1); RD_B(fb[2], 0, 0, 2); SB();
     int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
-        RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+    if constexpr (STAGES == 2) {
+        for (; kt + 1 < nk; kt += 2) {
+            RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+            RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+        }
+        if (kt < nk) RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+    } else {
+        // panel p waits in register set p mod 3; the LDS buffer alternates every step, so its
+        // index is a variable here (three steps flip it once)
+        int pb = 0;
+        for (; kt + 2 < nk; kt += 3) {
+            RF_STEP(pb, la1, lb1, la0, lb0, kt + 3);
+            RF_STEP(pb ^ 1, la2, lb2, la1, lb1, kt + 4);
+            RF_STEP(pb, la0, lb0, la2, lb2, kt + 5);
+            pb ^= 1;
+        }
+        if (kt < nk) RF_STEP(pb, la1, lb1, la0, lb0, kt + 3);
+        if (kt + 1 < nk) RF_STEP(pb ^ 1, la2, lb2, la1, lb1, kt + 4);
     }
-    if (kt < nk) RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
 #undef K0_OF
 #undef ROW_A
 #undef ROW_B
@@ -278,7 +328,7 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
     const int lr = lane & 31, lg = lane >> 5;
     char* stage = smem + PANEL_BYTES + wave * STAGE_BYTES;
     const int gcol0 = col0 + wn * 96;
-    const int grow0 = row0 + wm * 64;
+    const int grow0 = row0 + wm * WROWS;
     const int sr = lr & (ROWS - 1);                              // staged row of this lane
     const bool has_bias = BIAS && g.epilogue != PTJ_EPI_NONE;
     const bool act = ACT && g.epilogue == PTJ_EPI_BIAS_GELU;
@@ -318,7 +368,7 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
     }
     OUT* gbase = dst + (int64_t)(grow0 + rrow) * dst_rs + gcol0 + rch * V;
 #pragma unroll
-    for (int pass = 0; pass < 64 / ROWS; ++pass) {
+    for (int pass = 0; pass < WROWS / ROWS; ++pass) {
         const int tm = pass * ROWS / 32;
         const bool mine = ROWS == 32 || (lr >> 4) == (pass & 1);
 #pragma unroll
@@ -462,9 +512,10 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
     const T* B = (const T*)g.b;
     char* sA = smem;
     char* sB = smem + 2 * A_BYTES;
-    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1;
-    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1;
+    TileLoader<T, AMODE, BM, GEMM_THREADS, true> la0, la1, la2;
+    TileLoader<T, BMODE, BN, GEMM_THREADS, true> lb0, lb1, lb2;
     typename Frag<T>::type fa[2][TM], fb[TN], fx[TN];
+    int pb = 0;   // LDS buffer that holds the current tile's first panel (three staging sets only)
     // item -> tile origin, first contraction element, number of panels (even), partial tile
 #define STREAM_ITEM(ITEM, ROW0, COL0, KBEG, NK, PART)                                                    \
     do {                                                                                                 \
@@ -492,11 +543,15 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
         const int tid = fresh_tid();
         const int lane = tid & 63, wave = tid >> 6;
         const int lr = lane & 31, lg = lane >> 5;
-        const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
+        const int arow = (wave / WAVES_N) * WROWS + lr, brow = (wave % WAVES_N) * 96 + lr;
         la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, kbeg, tid, g.n);
         lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, kbeg, tid, g.m);
         la1.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, kbeg + BK, tid, g.n);
         lb1.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, kbeg + BK, tid, g.m);
+        if constexpr (STAGES == 3) {
+            la2.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, kbeg + 2 * BK, tid, g.n);
+            lb2.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, kbeg + 2 * BK, tid, g.m);
+        }
         la0.store(sA, tid);
         lb0.store(sB, tid);
         __syncthreads();
@@ -519,13 +574,24 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
             const int tid = fresh_tid();
             const int lane = tid & 63, wave = tid >> 6;
             const int lr = lane & 31, lg = lane >> 5;
-            const int arow = (wave / WAVES_N) * 64 + lr, brow = (wave % WAVES_N) * 96 + lr;
+            const int arow = (wave / WAVES_N) * WROWS + lr, brow = (wave % WAVES_N) * 96 + lr;
 #define K0_OF(KT) ((KT) < nk ? kbeg + (KT) * BK : nkbeg + ((KT) - nk) * BK)
 #define ROW_A(KT) ((KT) < nk ? row0 : nrow0)
 #define ROW_B(KT) ((KT) < nk ? col0 : ncol0)
-            for (int kt = 0; kt < nk; kt += 2) {
-                RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
-                RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+            if constexpr (STAGES == 2) {
+                for (int kt = 0; kt < nk; kt += 2) {
+                    RF_STEP(0, la1, lb1, la0, lb0, kt + 2);
+                    RF_STEP(1, la0, lb0, la1, lb1, kt + 3);
+                }
+            } else {
+                // nk is a multiple of 3 here: every tile starts with its panels 0, 1, 2 in LDS
+                // buffer pb, set 1 and set 2
+                for (int kt = 0; kt < nk; kt += 3) {
+                    RF_STEP(pb, la1, lb1, la0, lb0, kt + 3);
+                    RF_STEP(pb ^ 1, la2, lb2, la1, lb1, kt + 4);
+                    RF_STEP(pb, la0, lb0, la2, lb2, kt + 5);
+                    pb ^= 1;
+                }
             }
 #undef K0_OF
 #undef ROW_A
@@ -751,7 +817,8 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     int64_t work = (int64_t)num_m * num_n * splits;
     if (g.tail_splits > 1) work = g.tail_first + ((int64_t)num_m * num_n - g.tail_first) * g.tail_splits;
-    dim3 grid((unsigned)(work < NUM_CUS ? work : NUM_CUS)), block(GEMM_THREADS);
+    const int cus = num_cus();
+    dim3 grid((unsigned)(work < cus ? work : cus)), block(GEMM_THREADS);
 #define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD>), grid, block, 0, st, g)
     switch (am * 3 + bm) {
         case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
@@ -794,7 +861,7 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
 // of one per CU, a workgroup costs a fixed prologue/epilogue plus a per-panel time, and
 // every split writes and re-reads an fp32 copy of C.
 int choose_splits(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes) {
-    constexpr int CUS = 256;
+    const int CUS = num_cus();
     constexpr double T_FIXED_US = 6.0, T_PANEL_US = 1.6, BYTES_PER_US = 4.0e6;
     const int64_t tiles = ((n + BM - 1) / BM) * ((m + BN - 1) / BN);
     const int bk = BKB / elt;
@@ -818,7 +885,7 @@ int choose_splits(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes) {
 // for a whole tile time; they are cut into `*splits` K slices each so that the last round
 // fills the chip and takes 1/splits of a tile time.  Returns the workspace bytes (0 = off).
 size_t choose_tail_split(int64_t n, int64_t m, int64_t k, int elt, size_t ws_bytes, int* first, int* splits, int* kps) {
-    constexpr int CUS = 256;
+    const int CUS = num_cus();
     const int64_t tiles = ((n + BM - 1) / BM) * ((m + BN - 1) / BN);
     const int bk = BKB / elt;
     const int64_t panels = k / bk;
@@ -899,7 +966,7 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     }
     g.partial = (splits > 1 || g.tail_splits > 1) ? (float*)workspace : nullptr;
     // streamed tiles need whole, evenly many K panels (the two-step loop body) and vector-aligned outputs
-    g.stream = (splits == 1 && g.vec_out && k >= 2 * bk && k % (2 * bk) == 0) ? 1 : 0;
+    g.stream = (splits == 1 && g.vec_out && k >= STAGES * bk && k % (STAGES * bk) == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
 }
