@@ -223,6 +223,37 @@ def c4_leg(torch, mt, lo, dtype):
             "ce_GBs_3numel": round(3 * N * V * e / (t_ce * 1e-3) / 1e9, 1)}
 
 
+def only_leg(torch, mt, lo, which, c):
+    """A few launches of one kernel family at the training step's shapes (bf16), for counter passes."""
+    dev = "cuda:0"
+    B, T, H, D, F, V = c["B"], c["T"], c["H"], c["D"], c["F"], c["V"]
+    N, dh = B * T, c["D"] // c["H"]
+    bf = torch.bfloat16
+    if which == "attn":
+        qkv = torch.randn(B, H, 3, T, dh, device=dev).to(bf)
+        dO = torch.randn(B, H, T, dh, device=dev).to(bf)
+        q, k, v = qkv.unbind(2)
+        for _ in range(3):
+            o, ms_, ls_ = mt.attn_fwd_t(q, k, v, None, True, 5)
+            mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, None, True, 5)
+    elif which == "gemm":
+        x = torch.randn(N, D, device=dev).to(bf)
+        w1 = torch.randn(F, D, device=dev).to(bf)
+        dy = torch.randn(N, F, device=dev).to(bf)
+        for _ in range(3):
+            mt.matmul_t(x, w1.t())          # forward product   [N,D] x [D,F]   (both operands K-major)
+            mt.matmul_t(dy, w1)             # dX product        [N,F] x [F,D]   (B transposed on load)
+            mt.matmul_t(dy.t(), x)          # dW product        [F,N] x [N,D]   (both transposed, K split)
+    else:
+        logits = mt._padded_logits(N, V, bf, dev)
+        lab = torch.randint(0, V, (N,), device=dev)
+        for _ in range(3):
+            logits.normal_()
+            lo.t_avg_cross_entropy_loss_bkwd3_t(lab, logits, inplace=True, want_pred=True, want_colsum=True)
+    torch.cuda.synchronize()
+    print(json.dumps({"only": which, "launch_sets": 3}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -232,6 +263,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the legs of baseline configurations 2, 3 and 4")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run one plain 1 GiB device copy first (reference reading for FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--only", choices=["attn", "gemm", "ce"], default=None,
+                    help="run just a few launches of one kernel family at the step's shapes and exit "
+                         "(short programs for rocprofv3 counter passes)")
     ap.add_argument("--steps-only", action="store_true",
                     help="only the timed training steps (for profiling): no per-kernel legs, no CPU leg")
     args = ap.parse_args()
@@ -250,6 +284,10 @@ def main():
     torch.cuda.set_device(0)
     c = CFG
     B, T, V = c["B"], c["T"], c["V"]
+
+    if args.only is not None:
+        only_leg(torch, mt, lo, args.only, c)
+        return
 
     master, shadow, moments, wd_mask = make_state(torch, lo, c, dev)
     tok_gen = torch.Generator().manual_seed(99)
