@@ -446,20 +446,51 @@ def _aligned_view(t):
     return t
 
 
+ATTN_DH = 64   # head dimension of the attention kernels
+
+
+def _pad_heads(t, scale=None):
+    """[..., dh] -> [..., 64] with zero columns (optionally times `scale`): zero columns add
+    nothing to q.k and produce zero output columns."""
+    out = torch.zeros(t.shape[:-1] + (ATTN_DH,), dtype=t.dtype, device=t.device)
+    out[..., :t.shape[-1]] = t if scale is None else t * scale
+    return out
+
+
 def t_scaled_dot_prod_attn_fwd3_t(qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
-    """qkv [B,H,3,T,dh], mask [B,T,T] bool -> (O [B,H,T,dh], [ms, ls, O])."""
-    q, k, v = (_aligned_view(t) for t in torch.unbind(qkv, dim=2))
+    """qkv [B,H,3,T,dh], mask [B,T,T] bool -> (O [B,H,T,dh], [ms, ls, O]).
+
+    The kernels are written for dh = 64.  Smaller head sizes (the reference takes any power of
+    two, model_triton.py:716) are run on zero-padded copies: q is scaled by sqrt(64/dh) so that
+    the kernels' 1/sqrt(64) gives 1/sqrt(dh), and O is cut back to dh columns."""
     if train:
         assert p_gen_aux is not None
-    o, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux)
+    dh = qkv.shape[-1]
+    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
+    q, k, v = torch.unbind(qkv, dim=2)
+    if dh < ATTN_DH:
+        o, ms, ls = attn_fwd_t(_pad_heads(q, math.sqrt(ATTN_DH / dh)), _pad_heads(k), _pad_heads(v), mask, train,
+                               p_gen_aux)
+        o = o[..., :dh].contiguous()
+        return o, [ms, ls, o]
+    o, ms, ls = attn_fwd_t(_aligned_view(q), _aligned_view(k), _aligned_view(v), mask, train, p_gen_aux)
     return o, [ms, ls, o]
 
 
 def t_scaled_dot_prod_attn_bkwd3_t(dloss_dx, acts, qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
     """-> (dq, dk, dv), each [B,H,T,dh]."""
-    q, k, v = (_aligned_view(t) for t in torch.unbind(qkv, dim=2))
     ms, ls, o = acts
-    return attn_bwd_t(_aligned_view(dloss_dx), q, k, v, _aligned_view(o), ms, ls, mask, train, p_gen_aux)
+    dh = qkv.shape[-1]
+    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
+    q, k, v = torch.unbind(qkv, dim=2)
+    if dh < ATTN_DH:
+        f = math.sqrt(ATTN_DH / dh)
+        dq, dk, dv = attn_bwd_t(_pad_heads(dloss_dx), _pad_heads(q, f), _pad_heads(k), _pad_heads(v), _pad_heads(o), ms,
+                                ls, mask, train, p_gen_aux)
+        # q' = f q: dq = f dq'
+        return dq[..., :dh] * f, dk[..., :dh].contiguous(), dv[..., :dh].contiguous()
+    return attn_bwd_t(_aligned_view(dloss_dx), _aligned_view(q), _aligned_view(k), _aligned_view(v), _aligned_view(o), ms,
+                      ls, mask, train, p_gen_aux)
 
 
 # ----------------------------------------------------------------------------------
