@@ -70,6 +70,18 @@ struct AttnArgs {
 // ---- small device helpers -----------------------------------------------------------
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// max / sum of a value with its partner in the other half of the wavefront (lane ^ 32), the same
+// in both lanes: v_permlane32_swap exchanges the upper half of one register with the lower half
+// of another inside the vector ALU (no LDS round trip); with both registers holding v the two
+// results are {lo, lo} and {hi, hi}.
+__device__ __forceinline__ float max_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 // The 16-byte operand pieces of one 64-element row held in registers (lane half lg).
 template <typename T>
@@ -273,6 +285,7 @@ __global__ __launch_bounds__(256) void attn_pack_mask_kernel(const uint8_t* __re
 //      K tile gives each lane 32 score elements against 16 MFMAs = 512 cycles; every
 //      instruction per element counts, so masks and dropout are compiled in only where used)
 constexpr float NEG_RAW = -8e9f;          // masked raw score: NEG_RAW * (1/sqrt(64)) = -1e9
+constexpr float RESCALE_SLACK = 8.0f;     // forward: the reference point of the exponentials may lag the row maximum by 2^8
 constexpr float MASKED_BELOW = -1e8f;     // log2-domain row max below this = fully masked row
 
 // Causal / explicit-mask visibility of the lane's 16 elements of sub-tile j written into
@@ -350,7 +363,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
-    float m_run = NEG_RAW * sc, l_run = 0.f;
+    float m_run = NEG_RAW * sc, m_true = NEG_RAW * sc, l_run = 0.f;
     f32x16 o[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -398,26 +411,34 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[j][i]);
-            tmax = fmaxf(tmax, xor32(tmax));
-            const float m_new = fmaxf(m_run, tmax * sc);
-            const float alpha = fast_exp2(m_run - m_new);
+            tmax = max_xor32(tmax) * sc;
+            m_true = fmaxf(m_true, tmax);
+            // The exponentials are taken relative to m_run, which follows the true row maximum
+            // only when some row of the wavefront has outgrown it by more than 2^RESCALE_SLACK:
+            // softmax does not depend on the reference point, p stays below 2^RESCALE_SLACK, and
+            // the 32 rescaling multiplies of the accumulators are skipped on most tiles.  The
+            // saved statistics are converted to the true maximum at the end.
+            if (__builtin_amdgcn_ballot_w64(tmax > m_run + RESCALE_SLACK) != 0) {
+                const float m_new = fmaxf(m_run, tmax);
+                const float alpha = fast_exp2(m_run - m_new);
+                l_run *= alpha;
+                m_run = m_new;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+            }
             float p[2][16];
             float lsum = 0.f;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float e = fast_exp2(fmaf(s[j][i], sc, -m_new));
+                    const float e = fast_exp2(fmaf(s[j][i], sc, -m_run));
                     p[j][i] = e;
                     lsum += e;
                 }
-            lsum += xor32(lsum);
-            l_run = fmaf(l_run, alpha, lsum);
-            m_run = m_new;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+            l_run += sum_xor32(lsum);
             if constexpr (TRAIN) {
                 keep_apply<0>(p[0], kw);
                 keep_apply<1>(p[1], kw);
@@ -435,8 +456,9 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
         const float f = (TRAIN ? 1.0f : 0.9f) / l_run;
         store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, o, f, lg);
         if (lg == 0) {
-            a.ms[(int64_t)bh * a.T + query] = m_run < MASKED_BELOW ? NEG_NAT : m_run * LN2;
-            a.ls[(int64_t)bh * a.T + query] = l_run;
+            // statistics relative to the true row maximum: sum exp(s - m_true) = l_run 2^(m_run - m_true)
+            a.ms[(int64_t)bh * a.T + query] = m_true < MASKED_BELOW ? NEG_NAT : m_true * LN2;
+            a.ls[(int64_t)bh * a.T + query] = l_run * fast_exp2(m_run - m_true);
         }
     }
 }
@@ -571,9 +593,11 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                         float p = fast_exp2(fmaf(s[i], sc, -m4[b]));
                         if constexpr (!FOLD_L) p *= l4[b];
                         if constexpr (TRAIN) {
+                            // dS = P (keep ? dP : 0) - P delta = (keep ? P : 0) dP - P delta: the dropped
+                            // probability is needed anyway, so one select serves both products
                             const uint64_t km = keep_lane_mask_at(kw, j * 32 + g4 * 8 + b);
                             pd[i] = keep_select(p, km);
-                            ds[i] = p * (keep_select(dp[i], km) - d4[b]);
+                            ds[i] = fmaf(pd[i], dp[i], -(p * d4[b]));
                         } else {
                             pd[i] = 0.9f * p;
                             ds[i] = p * fmaf(dp[i], 0.9f, -d4[b]);
