@@ -38,6 +38,7 @@ extern "C" {
 #define PTJ_EPI_NONE 0
 #define PTJ_EPI_BIAS 1           /* C = A.B + bias[m]                       */
 #define PTJ_EPI_BIAS_GELU 2      /* C = gelu(A.B + bias[m])                 */
+#define PTJ_EPI_BIAS_GELU_DERIV 3 /* the same C; c_pre = gelu'(A.B + bias[m]) */
 
 int ptj_version(void);
 const char* ptj_last_error(void);
@@ -219,13 +220,30 @@ int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss
  * split along k: pass ptj_gemm_workspace_bytes(n, m, k, dtype) bytes; the split
  * partials are reduced in fixed order, so results are deterministic.  `c_pre`
  * (nullable, PTJ_EPI_BIAS_GELU only) additionally receives A.B + bias before the GELU:
- * the activation the backward needs (the reference recomputes it, model_triton.py:1415-1418). */
+ * the activation the backward needs (the reference recomputes it, model_triton.py:1415-1418).
+ * With PTJ_EPI_BIAS_GELU_DERIV `c_pre` (required) receives gelu'(A.B + bias) instead, taken from
+ * the fp32 accumulators with the exponential the GELU needs anyway: what the backward multiplies
+ * the incoming gradient by (t_gelu_bkwd2_k, model_triton.py:274-294). */
 size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype);
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
              int64_t n, int64_t m, int64_t k,
              int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs,
              int epilogue, void* c_pre, int64_t c_pre_rs,
              void* workspace, size_t workspace_bytes, int dtype, void* stream);
+
+/* C[n,m] = round(A.B) * mul[n,m] element-wise, and colsum[m] = the column sums of the stored C:
+ * the product that carries a gradient back through the feed-forward block's second linear layer
+ * (t_proj_bkwd2_x, model_triton.py:495-508), the GELU backward (t_gelu_bkwd2_k, :274-294; `mul` =
+ * gelu' kept by PTJ_EPI_BIAS_GELU_DERIV) and the first layer's bias gradient (:426) in one
+ * launch plus a small fixed-order reduction.  A.B is rounded to the storage type before the
+ * multiplication, as when the product is stored and re-read.  Operands as for ptj_gemm; `mul`
+ * and C are row-major with row strides mul_rs / c_rs.  `workspace` must hold
+ * ptj_gemm_mul_colsum_workspace_bytes(n, m) bytes (one fp32 row of sums per 64 rows of C). */
+size_t ptj_gemm_mul_colsum_workspace_bytes(int64_t n, int64_t m);
+int ptj_gemm_mul_colsum(const void* a, const void* b, const void* mul, void* c, void* colsum,
+                        int64_t n, int64_t m, int64_t k,
+                        int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t mul_rs, int64_t c_rs,
+                        void* workspace, size_t workspace_bytes, int dtype, void* stream);
 
 /* ---- optimizer ----------------------------------------------------------- */
 

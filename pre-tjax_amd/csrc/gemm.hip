@@ -107,6 +107,11 @@ struct GemmArgs {
     int stream;           // no K split and K is a whole even number of panels: tiles are pipelined back to back
     int vec_out;          // every output (C, pre-activation, partials) and the bias allow aligned 16-byte rows
     int epilogue;
+    // gemm_kernel<..., MUL = true> only: C = round(A.B) * mul element-wise, and the column sums of the
+    // stored C over each block of 64 rows go to colpart[row / 64][m]
+    const void* mul;
+    int64_t mul_rs;
+    float* colpart;
 };
 
 // A run of K panels [kt0, kt1) of one C tile through the element-wise edge loader (tiles
@@ -340,13 +345,18 @@ constexpr int SMEM_BYTES = PANEL_BYTES + (GEMM_THREADS / 64) * STAGE_BYTES;
 // The write-back gives each row of a group to LPR consecutive lanes (64 or 128 contiguous
 // bytes per row, 16 or 8 rows per store instruction).
 // BIAS: add g.bias here (false when the accumulators were started from the bias).
-// ACT: apply the GELU when the epilogue asks for it.
+// ACT: 1 = apply the GELU when the epilogue asks for it (both GELU epilogues); 2 = the GELU's
+// derivative instead (the second output of PTJ_EPI_BIAS_GELU_DERIV).  One pass that evaluates the
+// exponential once for both outputs was built as well: holding the second output of a pass in
+// registers costs more in spills than the second evaluation.
+// MUL: the stored value is round(acc) * g.mul[row, col], and its column sums over the
+// wavefront's 64 rows are written to g.colpart (fixed order: deterministic).
 // FULL: the tile lies inside C and dst / bias are vector-aligned, so the write-back is
 // straight-line 16-byte stores; otherwise every element is bounds-checked.  The two
 // variants are separate instantiations on purpose: when both appear behind one per-lane
 // condition the compiler merges them into partial (12 + 2 + 2 byte) stores.  The global
 // stores are not waited for.
-template <typename OUT, typename T, bool BIAS, bool ACT, bool FULL>
+template <typename OUT, typename T, bool BIAS, int ACT, bool FULL, bool MUL = false>
 __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
                                                  int row0, int col0, OUT* __restrict__ dst, int64_t dst_rs) {
     constexpr int RB = 96 * (int)sizeof(OUT);                    // bytes per staged row
@@ -365,7 +375,8 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
     const int grow0 = row0 + wm * WROWS;
     const int sr = lr & (ROWS - 1);                              // staged row of this lane
     const bool has_bias = BIAS && g.epilogue != PTJ_EPI_NONE;
-    const bool act = ACT && g.epilogue == PTJ_EPI_BIAS_GELU;
+    const bool act = ACT == 1 && (g.epilogue == PTJ_EPI_BIAS_GELU || g.epilogue == PTJ_EPI_BIAS_GELU_DERIV);
+    static_assert(!MUL || (WROWS == 64 && !BIAS && ACT == 0 && sizeof(OUT) == sizeof(T)), "MUL epilogue");
 
     // bias of this lane's 12 column quads
     float bias[TN * 4][4];
@@ -401,10 +412,31 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
         rbase[h] = stage + r * RB + ((rch ^ ((r >> KS) & (LPR - 1))) << 4);
     }
     OUT* gbase = dst + (int64_t)(grow0 + rrow) * dst_rs + gcol0 + rch * V;
+    // MUL: the multiplier element beside every stored element, and this lane's column sums: its V
+    // columns of each 32-column group over the rows it writes
+    const OUT* mbase = nullptr;
+    float cs[3][V];
+    if constexpr (MUL) {
+        mbase = (const OUT*)g.mul + (int64_t)(grow0 + rrow) * g.mul_rs + gcol0 + rch * V;
+#pragma unroll
+        for (int g3 = 0; g3 < 3; ++g3)
+#pragma unroll
+            for (int e = 0; e < V; ++e) cs[g3][e] = 0.f;
+    }
 #pragma unroll
     for (int pass = 0; pass < WROWS / ROWS; ++pass) {
         const int tm = pass * ROWS / 32;
         const bool mine = ROWS == 32 || (lr >> 4) == (pass & 1);
+        // the multipliers of this pass are requested before the block is staged
+        Pack<OUT, V> mv[ROWS / RPI][3];
+        if constexpr (MUL && FULL) {
+#pragma unroll
+            for (int h = 0; h < ROWS / RPI; ++h)
+#pragma unroll
+                for (int g3 = 0; g3 < 3; ++g3)
+                    mv[h][g3] = *reinterpret_cast<const Pack<OUT, V>*>(mbase + (int64_t)(pass * ROWS + h * RPI) * g.mul_rs +
+                                                                        g3 * 32);
+        }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -416,11 +448,15 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
 #pragma unroll
                     for (int e = 0; e < 4; ++e) o[e] += bias[tn * 4 + i4][e];
                 }
-                if constexpr (ACT) {
+                if constexpr (ACT == 1) {
                     if (act) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) o[e] = gelu_f(o[e]);
                     }
+                }
+                if constexpr (ACT == 2) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = gelu_grad_f(o[e]);
                 }
                 if (ROWS == 32 || mine) store_vec<OUT, 4>(reinterpret_cast<OUT*>(wrow + tn * (LPR * 16) + woff[i4]), o);
             }
@@ -430,20 +466,55 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
 #pragma unroll
             for (int g3 = 0; g3 < 3; ++g3) {
                 const int r = pass * ROWS + h * RPI;             // block row of the instruction's first row
-                const Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(rbase[h] + g3 * (LPR * 16));
+                Pack<OUT, V> val = *reinterpret_cast<const Pack<OUT, V>*>(rbase[h] + g3 * (LPR * 16));
                 OUT* p = gbase + (int64_t)r * dst_rs + g3 * 32;
                 if constexpr (FULL) {
+                    if constexpr (MUL) {
+#pragma unroll
+                        for (int e = 0; e < V; ++e) {
+                            val.v[e] = from_f32<OUT>(to_f32(val.v[e]) * to_f32(mv[h][g3].v[e]));
+                            cs[g3][e] += to_f32(val.v[e]);
+                        }
+                    }
                     *reinterpret_cast<Pack<OUT, V>*>(p) = val;
                 } else {
                     if (grow0 + r + rrow < g.n) {
                         const int gcol = gcol0 + g3 * 32 + rch * V;
 #pragma unroll
                         for (int e = 0; e < V; ++e)
-                            if (gcol + e < g.m) p[e] = val.v[e];
+                            if (gcol + e < g.m) {
+                                if constexpr (MUL) {
+                                    val.v[e] = from_f32<OUT>(to_f32(val.v[e]) *
+                                                             to_f32(mbase[(int64_t)r * g.mul_rs + g3 * 32 + e]));
+                                    cs[g3][e] += to_f32(val.v[e]);
+                                }
+                                p[e] = val.v[e];
+                            }
                     }
                 }
             }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    }
+    if constexpr (MUL) {
+        // lanes with equal (lane mod LPR) hold the same columns for different rows: butterfly over
+        // the row bits, then the lanes of row 0 write the wavefront's 96 sums
+#pragma unroll
+        for (int g3 = 0; g3 < 3; ++g3)
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float v = cs[g3][e];
+#pragma unroll
+                for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+                cs[g3][e] = v;
+            }
+        if (rrow == 0 && grow0 < g.n) {
+            float* cp = g.colpart + (int64_t)(grow0 / 64) * g.m + gcol0 + rch * V;
+#pragma unroll
+            for (int g3 = 0; g3 < 3; ++g3)
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (FULL || gcol0 + g3 * 32 + rch * V + e < g.m) cp[g3 * 32 + e] = cs[g3][e];
+        }
     }
 }
 
@@ -473,22 +544,33 @@ __device__ __forceinline__ void tile_origin(int pid, int total, int num_m, int n
 // Bias / GELU are applied in registers, the block is converted to the output type,
 // staged in the wave-private LDS area and written back as 16-byte vectors that run
 // along whole 96-column rows.  Only wave-local ordering is needed.
-template <typename T, bool BIAS, bool SPLIT = true>
+template <typename T, bool BIAS, bool SPLIT = true, bool MUL = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, const f32x16 (&acc)[TN][TM], char* __restrict__ smem,
                                               int row0, int col0, int z) {
     const bool full = row0 + BM <= g.n && col0 + BN <= g.m && g.vec_out;
-    if (SPLIT && g.partial != nullptr) {
+    if constexpr (MUL) {
+        if (full) gemm_store_block<T, T, false, 0, true, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        else gemm_store_block<T, T, false, 0, false, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+    } else if (SPLIT && g.partial != nullptr) {
         float* part = g.partial + (int64_t)z * g.n * (int64_t)g.m;
-        if (full) gemm_store_block<float, T, false, false, true>(g, acc, smem, row0, col0, part, g.m);
-        else gemm_store_block<float, T, false, false, false>(g, acc, smem, row0, col0, part, g.m);
+        if (full) gemm_store_block<float, T, false, 0, true>(g, acc, smem, row0, col0, part, g.m);
+        else gemm_store_block<float, T, false, 0, false>(g, acc, smem, row0, col0, part, g.m);
     } else if (full) {
-        if (g.c_aux != nullptr)
-            gemm_store_block<T, T, BIAS, false, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
-        gemm_store_block<T, T, BIAS, true, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        if (g.c_aux != nullptr) {
+            if (g.epilogue == PTJ_EPI_BIAS_GELU_DERIV)
+                gemm_store_block<T, T, BIAS, 2, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+            else
+                gemm_store_block<T, T, BIAS, 0, true>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+        }
+        gemm_store_block<T, T, BIAS, 1, true>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
     } else {
-        if (g.c_aux != nullptr)
-            gemm_store_block<T, T, BIAS, false, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
-        gemm_store_block<T, T, BIAS, true, false>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
+        if (g.c_aux != nullptr) {
+            if (g.epilogue == PTJ_EPI_BIAS_GELU_DERIV)
+                gemm_store_block<T, T, BIAS, 2, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+            else
+                gemm_store_block<T, T, BIAS, 0, false>(g, acc, smem, row0, col0, (T*)g.c_aux, g.c_aux_rs);
+        }
+        gemm_store_block<T, T, BIAS, 1, false>(g, acc, smem, row0, col0, (T*)g.c, g.c_rs);
     }
 }
 
@@ -501,7 +583,7 @@ __device__ __forceinline__ void load_bias_quads(const GemmArgs& g, int col0, Pac
     const int lg = (tid & 63) >> 5, wn = (tid >> 6) % WAVES_N;
     const int gcol0 = col0 + wn * 96 + lg * 4;
     const T* bias = (const T*)g.bias;
-    if (zero || g.epilogue == PTJ_EPI_NONE) {
+    if (zero || g.epilogue == PTJ_EPI_NONE || bias == nullptr) {
 #pragma unroll
         for (int q = 0; q < TN * 4; ++q)
 #pragma unroll
@@ -534,7 +616,7 @@ __device__ __forceinline__ void load_bias_quads(const GemmArgs& g, int col0, Pac
 // loads are in flight.  A workgroup without a next tile re-fetches its own first panels.
 // The accumulators start from the bias (loaded while the previous tile's epilogue runs)
 // instead of zero, so the epilogue neither waits for bias loads nor adds them.
-template <typename T, int AMODE, int BMODE, bool CLAMP>
+template <typename T, int AMODE, int BMODE, bool CLAMP, bool MUL>
 __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict__ smem) {
     constexpr int BK = BKB / (int)sizeof(T);
     constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
@@ -632,8 +714,8 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
 #undef ROW_B
         }
         load_bias_quads<T, CLAMP>(g, ncol0, braw, npart != nullptr);
-        if (part != nullptr) gemm_store_block<float, T, false, false, true>(g, acc, smem, 0, 0, part, BN);
-        else gemm_epilogue<T, false, false>(g, acc, smem, row0, col0, 0);
+        if (part != nullptr) gemm_store_block<float, T, false, 0, true>(g, acc, smem, 0, 0, part, BN);
+        else gemm_epilogue<T, false, false, MUL>(g, acc, smem, row0, col0, 0);
         if (!more) break;
         item = nitem;
         row0 = nrow0;
@@ -661,15 +743,15 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
 // Persistent kernel: workgroup b handles work items b, b + gridDim.x, ... where an item is
 // one (C tile, K split) pair; the stores of a finished tile drain while the next tile's
 // panels are loaded and multiplied.
-template <typename T, int AMODE, int BMODE>
+template <typename T, int AMODE, int BMODE, bool MUL = false>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g) {
     constexpr int BK = BKB / (int)sizeof(T);
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
     constexpr bool VECTOR_OK = AMODE != GENERIC && BMODE != GENERIC;
     if constexpr (VECTOR_OK) {
         if (g.stream) {
-            if (g.n % BM == 0 && g.m % BN == 0) gemm_stream<T, AMODE, BMODE, false>(g, smem);
-            else gemm_stream<T, AMODE, BMODE, true>(g, smem);
+            if (g.n % BM == 0 && g.m % BN == 0) gemm_stream<T, AMODE, BMODE, false, MUL>(g, smem);
+            else gemm_stream<T, AMODE, BMODE, true, MUL>(g, smem);
             return;
         }
     }
@@ -740,7 +822,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void gemm_kernel(const GemmArgs g)
         } else {
             gemm_run<T, AMODE, BMODE>(g, acc, smem, row0, col0, kbeg, kend, 0, nk);
         }
-        if (tail_part != nullptr) gemm_store_block<float, T, false, false, true>(g, acc, smem, 0, 0, tail_part, BN);
+        if constexpr (MUL) gemm_epilogue<T, false, false, true>(g, acc, smem, row0, col0, 0);
+        else if (tail_part != nullptr) gemm_store_block<float, T, false, 0, true>(g, acc, smem, 0, 0, tail_part, BN);
         else if (g.tail_splits > 1) gemm_epilogue<T, true, false>(g, acc, smem, row0, col0, z);
         else gemm_epilogue<T, true, true>(g, acc, smem, row0, col0, z);
     }
@@ -758,8 +841,9 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
         for (int z = 0; z < splits; ++z) s += partial[z * total + i];
         const int row = (int)(i / m), col = (int)(i - (int64_t)row * m);
         if (epilogue != PTJ_EPI_NONE) s += to_f32(bias[col]);
-        if (c_aux != nullptr) c_aux[(int64_t)row * c_aux_rs + col] = from_f32<T>(s);
-        if (epilogue == PTJ_EPI_BIAS_GELU) s = gelu_f(s);
+        if (c_aux != nullptr)
+            c_aux[(int64_t)row * c_aux_rs + col] = from_f32<T>(epilogue == PTJ_EPI_BIAS_GELU_DERIV ? gelu_grad_f(s) : s);
+        if (epilogue == PTJ_EPI_BIAS_GELU || epilogue == PTJ_EPI_BIAS_GELU_DERIV) s = gelu_f(s);
         c[(int64_t)row * c_rs + col] = from_f32<T>(s);
     }
 }
@@ -784,13 +868,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const float* _
             for (int e = 0; e < 4; ++e) s[e] += to_f32(b.v[e]);
         }
         Pack<T, 4> o;
+        const bool deriv = epilogue == PTJ_EPI_BIAS_GELU_DERIV;
         if (c_aux != nullptr) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o.v[e] = from_f32<T>(s[e]);
+            for (int e = 0; e < 4; ++e) o.v[e] = from_f32<T>(deriv ? gelu_grad_f(s[e]) : s[e]);
             *reinterpret_cast<Pack<T, 4>*>(c_aux + (int64_t)row * c_aux_rs + col) = o;
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o.v[e] = from_f32<T>(epilogue == PTJ_EPI_BIAS_GELU ? gelu_f(s[e]) : s[e]);
+        for (int e = 0; e < 4; ++e)
+            o.v[e] = from_f32<T>(epilogue == PTJ_EPI_BIAS_GELU || deriv ? gelu_f(s[e]) : s[e]);
         *reinterpret_cast<Pack<T, 4>*>(c + (int64_t)row * c_rs + col) = o;
     }
 }
@@ -823,10 +909,11 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const GemmArgs g)
         T* ca = g.c_aux != nullptr ? (T*)g.c_aux + (int64_t)row * g.c_aux_rs + col : nullptr;
         T* cc = (T*)g.c + (int64_t)row * g.c_rs + col;
         Pack<T, 4> pre, out;
+        const bool deriv = g.epilogue == PTJ_EPI_BIAS_GELU_DERIV;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            pre.v[e] = from_f32<T>(s[e]);
-            out.v[e] = from_f32<T>(g.epilogue == PTJ_EPI_BIAS_GELU ? gelu_f(s[e]) : s[e]);
+            pre.v[e] = from_f32<T>(deriv ? gelu_grad_f(s[e]) : s[e]);
+            out.v[e] = from_f32<T>(g.epilogue == PTJ_EPI_BIAS_GELU || deriv ? gelu_f(s[e]) : s[e]);
         }
         if (whole && g.vec_out) {
             if (ca != nullptr) *reinterpret_cast<Pack<T, 4>*>(ca) = pre;
@@ -851,7 +938,53 @@ int pick_mode(const void* p, int64_t s_row, int64_t s_k) {
     return GENERIC;
 }
 
+// Second stage of the MUL epilogue: out[col] = sum over the 64-row blocks of colpart[block][col].  A
+// workgroup owns 64 columns; its four wavefronts take the blocks b = w, w + 4, ... (independent,
+// coalesced loads, eight in flight) and their sums are combined in wavefront order: the order of
+// the additions is fixed.
 template <typename T>
+__global__ __launch_bounds__(256) void gemm_colpart_reduce_kernel(const float* __restrict__ colpart, int blocks, int m,
+                                                                   T* __restrict__ out) {
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int col = blockIdx.x * 64 + lane;
+    float s = 0.f;
+    if (col < m) {
+        int b = w;
+        for (; b + 28 < blocks; b += 32) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = colpart[(int64_t)(b + 4 * u) * m + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; b < blocks; b += 4) s += colpart[(int64_t)b * m + col];
+    }
+    part[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && col < m) out[col] = from_f32<T>((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
+}
+
+// The multiplying epilogue as a pass of its own, for operand layouts the GEMM reads element by
+// element: C = round(C * mul) in place and the column sums of the result per block of 64 rows.
+// One thread per column of a row block.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_mul_colpart_kernel(T* __restrict__ c, int64_t c_rs, const T* __restrict__ mul,
+                                                                int64_t mul_rs, int n, int m, float* __restrict__ colpart) {
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    const int rb = blockIdx.y;
+    if (col >= m) return;
+    const int r1 = (rb + 1) * 64 < n ? (rb + 1) * 64 : n;
+    float s = 0.f;
+    for (int r = rb * 64; r < r1; ++r) {
+        const T v = from_f32<T>(to_f32(c[(int64_t)r * c_rs + col]) * to_f32(mul[(int64_t)r * mul_rs + col]));
+        c[(int64_t)r * c_rs + col] = v;
+        s += to_f32(v);
+    }
+    colpart[(int64_t)rb * m + col] = s;
+}
+
+template <typename T, bool MUL = false>
 int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     const int am = pick_mode<T>(g.a, g.a_row, g.a_k), bm = pick_mode<T>(g.b, g.b_row, g.b_k);
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
@@ -859,17 +992,28 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     if (g.tail_splits > 1) work = g.tail_first + ((int64_t)num_m * num_n - g.tail_first) * g.tail_splits;
     const int cus = num_cus();
     dim3 grid((unsigned)(work < cus ? work : cus)), block(GEMM_THREADS);
-#define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD>), grid, block, 0, st, g)
-    switch (am * 3 + bm) {
-        case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
-        case 1: GEMM_LAUNCH(KMAJOR, MNMAJOR); break;
-        case 2: GEMM_LAUNCH(KMAJOR, GENERIC); break;
-        case 3: GEMM_LAUNCH(MNMAJOR, KMAJOR); break;
-        case 4: GEMM_LAUNCH(MNMAJOR, MNMAJOR); break;
-        case 5: GEMM_LAUNCH(MNMAJOR, GENERIC); break;
-        case 6: GEMM_LAUNCH(GENERIC, KMAJOR); break;
-        case 7: GEMM_LAUNCH(GENERIC, MNMAJOR); break;
-        default: GEMM_LAUNCH(GENERIC, GENERIC); break;
+#define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD, MUL>), grid, block, 0, st, g)
+    if constexpr (MUL) {
+        // the multiplying epilogue exists for vector-loadable operands only (the caller checks)
+        switch (am * 3 + bm) {
+            case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
+            case 1: GEMM_LAUNCH(KMAJOR, MNMAJOR); break;
+            case 3: GEMM_LAUNCH(MNMAJOR, KMAJOR); break;
+            case 4: GEMM_LAUNCH(MNMAJOR, MNMAJOR); break;
+            default: return ptj_set_error(PTJ_ERR_INVALID, "gemm: operand layout without a multiplying epilogue");
+        }
+    } else {
+        switch (am * 3 + bm) {
+            case 0: GEMM_LAUNCH(KMAJOR, KMAJOR); break;
+            case 1: GEMM_LAUNCH(KMAJOR, MNMAJOR); break;
+            case 2: GEMM_LAUNCH(KMAJOR, GENERIC); break;
+            case 3: GEMM_LAUNCH(MNMAJOR, KMAJOR); break;
+            case 4: GEMM_LAUNCH(MNMAJOR, MNMAJOR); break;
+            case 5: GEMM_LAUNCH(MNMAJOR, GENERIC); break;
+            case 6: GEMM_LAUNCH(GENERIC, KMAJOR); break;
+            case 7: GEMM_LAUNCH(GENERIC, MNMAJOR); break;
+            default: GEMM_LAUNCH(GENERIC, GENERIC); break;
+        }
     }
 #undef GEMM_LAUNCH
     PTJ_CHECK_LAUNCH();
@@ -965,14 +1109,15 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
              void* workspace, size_t workspace_bytes, int dtype, void* stream) {
     PTJ_CHECK_ARG(n >= 0 && m >= 0 && k >= 0, "gemm: negative dimension");
     PTJ_CHECK_ARG(n < (1ll << 31) && m < (1ll << 31) && k < (1ll << 31), "gemm: dimension exceeds 31 bits");
-    PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_BIAS_GELU, "gemm: unknown epilogue %d", epilogue);
+    PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_BIAS_GELU_DERIV, "gemm: unknown epilogue %d", epilogue);
+    PTJ_CHECK_ARG(epilogue != PTJ_EPI_BIAS_GELU_DERIV || c_pre, "gemm: the derivative epilogue needs its second output");
     PTJ_CHECK_ARG(epilogue == PTJ_EPI_NONE || bias, "gemm: epilogue %d needs a bias", epilogue);
     PTJ_CHECK_ARG(dtype == PTJ_F32 || dtype == PTJ_BF16, "gemm: unknown dtype %d", dtype);
     if (n == 0 || m == 0) return PTJ_OK;
     PTJ_CHECK_ARG(c && (k == 0 || (a && b)), "gemm: null pointer");
     PTJ_CHECK_ARG(c_rs >= m, "gemm: c row stride %lld < m %lld", (long long)c_rs, (long long)m);
-    PTJ_CHECK_ARG(!c_pre || (epilogue == PTJ_EPI_BIAS_GELU && c_pre_rs >= m),
-                  "gemm: c_pre needs the bias+GELU epilogue and a row stride >= m");
+    PTJ_CHECK_ARG(!c_pre || ((epilogue == PTJ_EPI_BIAS_GELU || epilogue == PTJ_EPI_BIAS_GELU_DERIV) && c_pre_rs >= m),
+                  "gemm: c_pre needs a bias+GELU epilogue and a row stride >= m");
     const int elt = dtype == PTJ_BF16 ? 2 : 4;
     const int bk = BKB / elt;
     GemmArgs g;
@@ -984,6 +1129,7 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     g.c_aux = c_pre;
     g.c_aux_rs = c_pre_rs;
     g.epilogue = epilogue;
+    g.mul = nullptr; g.mul_rs = 0; g.colpart = nullptr;
     int splits = workspace ? choose_splits(n, m, k, elt, workspace_bytes) : 1;
     int64_t kps = k;
     if (splits > 1) {
@@ -1009,6 +1155,78 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     g.stream = (splits == 1 && g.vec_out && k >= STAGES * bk && k % (STAGES * bk) == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? gemm_impl<float>(g, splits, st) : gemm_impl<bf16>(g, splits, st);
+}
+
+size_t ptj_gemm_mul_colsum_workspace_bytes(int64_t n, int64_t m) {
+    if (n <= 0 || m <= 0) return 0;
+    return (size_t)((n + 63) / 64) * (size_t)m * sizeof(float);
+}
+
+int ptj_gemm_mul_colsum(const void* a, const void* b, const void* mul, void* c, void* colsum, int64_t n, int64_t m,
+                        int64_t k, int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t mul_rs, int64_t c_rs,
+                        void* workspace, size_t workspace_bytes, int dtype, void* stream) {
+    PTJ_CHECK_ARG(n >= 0 && m >= 0 && k >= 0, "gemm_mul_colsum: negative dimension");
+    PTJ_CHECK_ARG(n < (1ll << 31) && m < (1ll << 31) && k < (1ll << 31), "gemm_mul_colsum: dimension exceeds 31 bits");
+    PTJ_CHECK_ARG(dtype == PTJ_F32 || dtype == PTJ_BF16, "gemm_mul_colsum: unknown dtype %d", dtype);
+    if (m == 0) return PTJ_OK;
+    PTJ_CHECK_ARG(colsum, "gemm_mul_colsum: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const size_t need = ptj_gemm_mul_colsum_workspace_bytes(n, m);
+    if (n > 0) {
+        PTJ_CHECK_ARG(c && mul && (k == 0 || (a && b)), "gemm_mul_colsum: null pointer");
+        PTJ_CHECK_ARG(c_rs >= m && mul_rs >= m, "gemm_mul_colsum: row stride below m %lld", (long long)m);
+        if (!workspace || workspace_bytes < need)
+            return ptj_set_error(PTJ_ERR_WORKSPACE, "gemm_mul_colsum: workspace %zu < %zu bytes", workspace_bytes, need);
+        const int elt = dtype == PTJ_BF16 ? 2 : 4;
+        const int bk = BKB / elt;
+        GemmArgs g;
+        g.a = a; g.b = b; g.c = c; g.bias = nullptr;
+        g.n = (int)n; g.m = (int)m; g.k = (int)k;
+        g.a_row = a_rs; g.a_k = a_cs;
+        g.b_row = b_cs; g.b_k = b_rs;
+        g.c_rs = c_rs;
+        g.c_aux = nullptr; g.c_aux_rs = 0;
+        g.epilogue = PTJ_EPI_NONE;
+        g.mul = mul; g.mul_rs = mul_rs; g.colpart = (float*)workspace;
+        g.k_per_split = k > 0 ? (int)k : bk;
+        g.splits = 1;
+        g.tail_first = 0; g.tail_splits = 1; g.tail_kps = 0;
+        g.partial = nullptr;
+        const int64_t v = 16 / elt;
+        g.vec_out = (ptj_aligned16(c) && c_rs % v == 0 && ptj_aligned16(mul) && mul_rs % v == 0 && ptj_aligned16(workspace) &&
+                     m % 4 == 0) ? 1 : 0;
+        g.stream = (g.vec_out && k >= STAGES * bk && k % (STAGES * bk) == 0) ? 1 : 0;
+        const bool vector_operands =
+            dtype == PTJ_F32 ? (pick_mode<float>(a, g.a_row, g.a_k) != GENERIC && pick_mode<float>(b, g.b_row, g.b_k) != GENERIC)
+                             : (pick_mode<bf16>(a, g.a_row, g.a_k) != GENERIC && pick_mode<bf16>(b, g.b_row, g.b_k) != GENERIC);
+        if (vector_operands) {
+            const int rc = dtype == PTJ_F32 ? gemm_impl<float, true>(g, 1, st) : gemm_impl<bf16, true>(g, 1, st);
+            if (rc != PTJ_OK) return rc;
+        } else {
+            // plain product first, then the multiplication and the sums as a pass over C
+            g.mul = nullptr; g.colpart = nullptr;
+            const int rc = dtype == PTJ_F32 ? gemm_impl<float>(g, 1, st) : gemm_impl<bf16>(g, 1, st);
+            if (rc != PTJ_OK) return rc;
+            const dim3 grid2((unsigned)((m + 255) / 256), (unsigned)((n + 63) / 64));
+            if (dtype == PTJ_F32)
+                hipLaunchKernelGGL((gemm_mul_colpart_kernel<float>), grid2, dim3(256), 0, st, (float*)c, c_rs, (const float*)mul,
+                                   mul_rs, (int)n, (int)m, (float*)workspace);
+            else
+                hipLaunchKernelGGL((gemm_mul_colpart_kernel<bf16>), grid2, dim3(256), 0, st, (bf16*)c, c_rs, (const bf16*)mul,
+                                   mul_rs, (int)n, (int)m, (float*)workspace);
+            PTJ_CHECK_LAUNCH();
+        }
+    }
+    const int blocks = (int)((n + 63) / 64);
+    const dim3 grid((unsigned)((m + 63) / 64));
+    if (dtype == PTJ_F32)
+        hipLaunchKernelGGL((gemm_colpart_reduce_kernel<float>), grid, dim3(256), 0, st, (const float*)workspace, blocks,
+                           (int)m, (float*)colsum);
+    else
+        hipLaunchKernelGGL((gemm_colpart_reduce_kernel<bf16>), grid, dim3(256), 0, st, (const float*)workspace, blocks,
+                           (int)m, (bf16*)colsum);
+    PTJ_CHECK_LAUNCH();
+    return PTJ_OK;
 }
 
 }  // extern "C"

@@ -285,13 +285,14 @@ def colsum_t(x: torch.Tensor):
 # ----------------------------------------------------------------------------------
 # GEMM  (reference: model_triton.py:373-398 t_matmul_t, :1258-1313 t_tlayer_ffn_fwd_t)
 # ----------------------------------------------------------------------------------
-def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, pre_out=None):
+def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, pre_out=None, deriv_out=None):
     """``out[N,M] = a[N,K] @ b[K,M] (+ bias[M]) (tanh-GELU)`` on the MFMA GEMM kernel.
 
     `a` and `b` are 2-D tensors with arbitrary strides (``.t()`` views are consumed in
     place, never copied); `out`, if given, is a 2-D tensor with unit column stride
     (a column slice of a wider buffer is fine).  `pre_out` (with ``gelu=True``) also
-    receives ``a @ b + bias`` before the activation."""
+    receives ``a @ b + bias`` before the activation; `deriv_out` (instead) receives the
+    GELU's derivative there, which is all the backward pass needs of it."""
     require_gpu(a, b, bias, out)
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], (a.shape, b.shape)
     assert a.dtype == b.dtype
@@ -311,12 +312,35 @@ def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, 
     code = dtype_code(a)
     ws_bytes = lib().ptj_gemm_workspace_bytes(N, M, K, code)
     ws = _workspace(ws_bytes, a.device, "gemm") if ws_bytes else None
+    if deriv_out is not None:
+        assert pre_out is None, "one second output"
+        pre_out, epi = deriv_out, _lib.EPI_BIAS_GELU_DERIV
     if pre_out is not None:
         assert gelu and pre_out.shape == (N, M) and pre_out.dtype == a.dtype and pre_out.stride(1) == 1
     check(lib().ptj_gemm(ptr(a), ptr(b), ptr(out), ptr(bias), N, M, K, a.stride(0), a.stride(1), b.stride(0),
                          b.stride(1), out.stride(0), epi, ptr(pre_out), pre_out.stride(0) if pre_out is not None else 0,
                          ptr(ws), ws_bytes, code, stream()), "ptj_gemm")
     return out
+
+
+def matmul_mul_colsum_t(a: torch.Tensor, b: torch.Tensor, mul: torch.Tensor):
+    """``c = (a @ b) * mul`` element-wise and the column sums of c, from one GEMM launch whose
+    epilogue multiplies and sums (plus a small fixed-order reduction): with `mul` the GELU
+    derivative kept by the forward pass this is d(pre-activation) and the gradient of the bias
+    in front of the activation (model_triton.py:495-508, :274-294, :426).  Returns (c, sums)."""
+    require_gpu(a, b, mul)
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], (a.shape, b.shape)
+    N, K = a.shape
+    M = b.shape[1]
+    assert a.dtype == b.dtype == mul.dtype and mul.shape == (N, M) and (mul.stride(1) == 1 or M == 1)
+    out = torch.empty((N, M), dtype=a.dtype, device=a.device)
+    sums = torch.empty(M, dtype=a.dtype, device=a.device)
+    ws_bytes = lib().ptj_gemm_mul_colsum_workspace_bytes(N, M)
+    ws = _workspace(ws_bytes, a.device, "gemm_colsum") if ws_bytes else None
+    check(lib().ptj_gemm_mul_colsum(ptr(a), ptr(b), ptr(mul), ptr(out), ptr(sums), N, M, K, a.stride(0), a.stride(1),
+                                    b.stride(0), b.stride(1), mul.stride(0), out.stride(0), ptr(ws), ws_bytes,
+                                    dtype_code(a), stream()), "ptj_gemm_mul_colsum")
+    return out, sums
 
 
 def t_matmul_t(a: torch.Tensor, b: torch.Tensor):
@@ -342,19 +366,19 @@ def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
 
 def t_tlayer_ffn_bkwd2_t(dloss_dx, layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
     """VJP of the feed-forward block without saved activations (model_triton.py:1410-1428):
-    the first linear layer is recomputed (bias+GELU epilogue that also keeps the
-    pre-activation), then dW2, db2, d(mid), GELU backward with db1, dW1 and dx.
+    the first linear layer is recomputed (bias+GELU epilogue that also keeps the GELU's
+    derivative), then dW2, db2, d(mid) times that derivative with db1 from the same launch,
+    dW1 and dx.
     Returns (dx shaped like x, (dW1, db1, dW2, db2))."""
     assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU backward exists"
     w1, b1, w2, b2 = layer_params
     x2 = _rows2d(x)
     d2 = _rows2d(dloss_dx)
-    pre = torch.empty((x2.shape[0], w1.shape[0]), dtype=x2.dtype, device=x2.device)
-    mid = matmul_t(x2, w1.t(), b1, gelu=True, pre_out=pre)
+    dgelu = torch.empty((x2.shape[0], w1.shape[0]), dtype=x2.dtype, device=x2.device)
+    mid = matmul_t(x2, w1.t(), b1, gelu=True, deriv_out=dgelu)
     db2 = colsum_t(d2)
     dw2 = matmul_t(d2.t(), mid)
-    dmid = matmul_t(d2, w2)
-    dpre, db1 = t_gelu_bkwd2_colsum_t(dmid, pre)
+    dpre, db1 = matmul_mul_colsum_t(d2, w2, dgelu)
     dw1 = matmul_t(dpre.t(), x2)
     dx = matmul_t(dpre, w1)
     return dx.reshape(x.shape), (dw1, db1, dw2, db2)
@@ -577,8 +601,8 @@ def t_gpt2_tlayer_fwd3_t(layer_params, y, mask, train=True, p_gen_aux=None, h1=N
     _, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux[0], out=o4)
     a_out = matmul_t(o2, wo.t())
     x_mid, h2, keep1 = dropout_add_layernorm_t(a_out, x_in, (ln2g, ln2b), train, p_gen_aux[1], want_keep=True)
-    f1 = torch.empty((N, w1.shape[0]), dtype=y.dtype, device=y.device)
-    g1 = matmul_t(h2, w1.t(), b1, gelu=True, pre_out=f1)               # bias + GELU epilogue, both kept
+    f1 = torch.empty((N, w1.shape[0]), dtype=y.dtype, device=y.device)  # gelu'(h2 @ W1^T + b1)
+    g1 = matmul_t(h2, w1.t(), b1, gelu=True, deriv_out=f1)             # bias + GELU epilogue; its derivative kept
     f2 = matmul_t(g1, w2.t(), b2)
     if next_ln is not None:
         x_out, h_next, keep2 = dropout_add_layernorm_t(f2, x_mid, next_ln, train, p_gen_aux[2], want_keep=True)
@@ -613,8 +637,7 @@ def t_gpt2_tlayer_bkwd3_t(dloss_dx, acts, layer_params, y, mask, train=True, p_g
     d = dropped_in if dropped_in is not None else t_dropout_bkwd2_t(dloss_dx, None, train, p_gen_aux[2])
     db2 = db2_in if (db2_in is not None and dropped_in is not None) else colsum_t(d)
     dw2 = matmul_t(d.t(), g1)                                           # [D,F]
-    dg1 = matmul_t(d, w2)                                               # [N,F]
-    df1, db1 = t_gelu_bkwd2_colsum_t(dg1, f1)
+    df1, db1 = matmul_mul_colsum_t(d, w2, f1)                           # [N,F] = (d @ W2) * gelu', and its column sums
     dw1 = matmul_t(df1.t(), h2)                                         # [F,D]
     dh2 = matmul_t(df1, w1)                                             # [N,D]
     dx_mid, (dln2g, dln2b), d = layernorm_bkwd2_t(dh2, (ln2g, ln2b), x_mid, residual=dloss_dx,

@@ -167,3 +167,81 @@ def test_gemm_gelu_dual_output(mt, dtype):
     check(act, x, w.t(), dtype, bias=b, gelu=True)
     # the activation is computed from the unrounded pre-activation, exactly as the single-output epilogue
     assert torch.equal(act, mt.matmul_t(x.to(DEV), w.to(DEV).t(), b.to(DEV), gelu=True))
+
+
+def _gelu_deriv64(x64):
+    """gelu'(x) in fp64 through the oracle's backward with a unit incoming gradient."""
+    return ops.gelu_bkwd2(torch.ones_like(x64), x64)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,m,k", [(300, 260, 200), (512, 384, 128), (256, 192, 768), (64, 100, 4096)])
+def test_gemm_gelu_derivative_output(mt, dtype, n, m, k):
+    """Second output of the derivative epilogue = gelu'(a @ b + bias); first output unchanged.
+    Shapes: edge tiles, whole tiles on the pipelined path, and a long K that is split."""
+    g = gen(15 + n)
+    x, w, b = randn(g, n, k, dtype=dtype), randn(g, m, k, dtype=dtype, std=0.1), randn(g, m, dtype=dtype)
+    der = torch.empty(n, m, dtype=dtype, device=DEV)
+    act = mt.matmul_t(x.to(DEV), w.to(DEV).t(), b.to(DEV), gelu=True, deriv_out=der)
+    check(act, x, w.t(), dtype, bias=b, gelu=True)
+    assert torch.equal(act, mt.matmul_t(x.to(DEV), w.to(DEV).t(), b.to(DEV), gelu=True))
+    pre64 = f64(x) @ f64(w).t() + f64(b)
+    want = _gelu_deriv64(pre64)
+    # |gelu''| <= 1.1: the error of the pre-activation carries over, plus the output rounding
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    scale = f64(x).abs() @ f64(w).t().abs() + f64(b).abs()
+    bound = 1.2 * tol * scale + (1e-6 if dtype == torch.float32 else 4e-3 * want.abs() + 1e-6)
+    err = (f64(der) - want).abs()
+    assert not (err > bound).any(), (err / bound).max().item()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,m,k,layout", [(512, 384, 128, "nn"), (256, 192, 768, "nt"), (300, 260, 200, "nn"),
+                                          (130, 70, 96, "tn"), (1024, 768, 256, "nn"), (33, 5, 7, "nn"),
+                                          (64, 100, 4096, "nn")])
+def test_gemm_multiply_epilogue_with_column_sums(mt, dtype, n, m, k, layout):
+    """(a @ b) * mul and its column sums against fp64; the product is the stored, rounded a @ b
+    times mul, and the sums are those of the stored result."""
+    g = gen(16 + n + m)
+    a = randn(g, n, k, dtype=dtype) if layout[0] == "n" else randn(g, k, n, dtype=dtype).t()
+    b = randn(g, k, m, dtype=dtype, std=0.1) if layout[1] == "n" else randn(g, m, k, dtype=dtype, std=0.1).t()
+    mul = randn(g, n, m, dtype=dtype)
+    ad = (a.t().contiguous().to(DEV).t() if layout[0] == "t" else a.to(DEV))
+    bd = (b.t().contiguous().to(DEV).t() if layout[1] == "t" else b.to(DEV))
+    c, sums = mt.matmul_mul_colsum_t(ad, bd, mul.to(DEV))
+    assert c.shape == (n, m) and sums.shape == (m,) and c.dtype == dtype and sums.dtype == dtype
+    # element-wise: the rounded a @ b (same bound as the plain product, which may sum a long K in
+    # another order) times mul, rounded once more
+    a64, b64, m64 = f64(a), f64(b), f64(mul)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    bound = (tol * (a64.abs() @ b64.abs()) + (0 if dtype == torch.float32 else 4e-3 * (a64 @ b64).abs())) * m64.abs()
+    bound = bound + (1e-30 if dtype == torch.float32 else 4e-3 * (a64 @ b64 * m64).abs() + 1e-6)
+    err = (f64(c) - a64 @ b64 * m64).abs()
+    assert not (err > bound).any(), (err / bound).max().item()
+    if dtype == torch.bfloat16 and k <= 768:             # one summation order: bit-equal to the two-step form
+        plain = mt.matmul_t(ad, bd)
+        assert torch.equal(c, (plain.float() * mul.to(DEV).float()).to(dtype))
+    want_s = f64(c).sum(0)
+    mag = f64(c).abs().sum(0)
+    tol = 1e-6 if dtype == torch.float32 else 5e-3       # fp32 accumulation, output rounded to storage
+    assert ((f64(sums) - want_s).abs() <= tol * mag + 1e-30).all(), ((f64(sums) - want_s).abs() / (mag + 1e-30)).max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ffn_backward_through_the_fused_epilogues(mt, dtype):
+    """t_tlayer_ffn_bkwd2_t (derivative epilogue forward, multiply + column-sum epilogue backward)
+    against autograd of the fp64 restatement."""
+    g = gen(17)
+    N, D, F = 384, 192, 576
+    x = randn(g, N, D, dtype=dtype)
+    w1, b1 = randn(g, F, D, dtype=dtype, std=0.05), randn(g, F, dtype=dtype, std=0.1)
+    w2, b2 = randn(g, D, F, dtype=dtype, std=0.05), randn(g, D, dtype=dtype, std=0.1)
+    dy = randn(g, N, D, dtype=dtype)
+    leaves = [f64(t).requires_grad_() for t in (x, w1, b1, w2, b2)]
+    out = ops.gelu(leaves[0] @ leaves[1].t() + leaves[2]) @ leaves[3].t() + leaves[4]
+    want = torch.autograd.grad(out, leaves, f64(dy))
+    dx, (dw1, db1, dw2, db2) = mt.t_tlayer_ffn_bkwd2_t(dy.to(DEV), tuple(t.to(DEV) for t in (w1, b1, w2, b2)), x.to(DEV))
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for name, got, w in zip(("dx", "dw1", "db1", "dw2", "db2"), (dx, dw1, db1, dw2, db2), want):
+        rel = ((f64(got) - w).norm() / w.norm()).item()
+        assert got.shape == w.shape and rel < tol, (name, rel)
