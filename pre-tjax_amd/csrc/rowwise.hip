@@ -634,6 +634,18 @@ __global__ __launch_bounds__(RED_THREADS) void colsum_stage2_kernel(const float*
     if ((threadIdx.x >> 5) == 0 && c < cols) out[c] = from_f32<T>(r);
 }
 
+// Second stage for a few partial rows (wide tensors with few rows, e.g. the sum over the batch
+// that is the positional table's gradient): one thread per column, the partials added in order.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_stage2_few_kernel(const float* __restrict__ part, int nparts, int cols,
+                                                                 T* __restrict__ out) {
+    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += (int64_t)gridDim.x * 256) {
+        float s = 0.f;
+        for (int p = 0; p < nparts; ++p) s += part[(int64_t)p * cols + c];
+        out[c] = from_f32<T>(s);
+    }
+}
+
 // GELU backward with the column sums of its own output (the bias gradient of the linear
 // layer in front of the GELU).  A workgroup owns whole rows: `tpr` threads cover a row
 // (thread t the 16-byte vectors t, t + tpr, ... : contiguous accesses) and the workgroup
@@ -765,8 +777,15 @@ int colsum_impl(const void* x, void* out, void* ws, size_t ws_bytes, int64_t row
         hipLaunchKernelGGL((colsum_stage1_kernel<T, 1>), dim3(gx, splits), dim3(128), 0, st, (const T*)x, (float*)ws,
                            rows, (int)cols, xs, rps);
     PTJ_CHECK_LAUNCH();
-    hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
-                       (const float*)ws, splits, (int)cols, (T*)out);
+    if (splits <= 8) {
+        int64_t blocks = (cols + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL((colsum_stage2_few_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (const float*)ws, splits,
+                           (int)cols, (T*)out);
+    } else {
+        hipLaunchKernelGGL((colsum_stage2_kernel<T>), dim3((unsigned)((cols + 31) / 32)), dim3(RED_THREADS), 0, st,
+                           (const float*)ws, splits, (int)cols, (T*)out);
+    }
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
 }

@@ -37,7 +37,7 @@ def test_adamw_matches_oracle(lo, gdtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(16384, 768), (1000, 50257), (37, 101), (1, 8), (4, 6, 64)])
+@pytest.mark.parametrize("shape", [(16384, 768), (1000, 50257), (37, 101), (1, 8), (4, 6, 64), (16, 98304), (150, 20000)])
 def test_colsum(mt, dtype, shape):
     g = gen(4)
     x = randn(g, *shape, dtype=dtype)
