@@ -414,7 +414,8 @@ def main():
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "traffic_note": "bytes per GEMM launch at the L2 boundary (average over the launches of a step) from "
                                      "rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy, read from "
-                                     "profiles/%s; algorithmic minimum 145.2e6" % os.path.basename(GEMM_TRAFFIC_FILE),
+                                     "profiles/%s; algorithmic minimum %.4g" % (os.path.basename(GEMM_TRAFFIC_FILE),
+                                                                                 float((traffic_src or {}).get("algorithmic_bytes_per_launch", 0))),
                      "kernel": "gemm_kernel<bf16> (all %d launches of a step: fwd, dX, dW)" % (n_launch // args.steps),
                      "avg_launch_ms": round(gemm_ms / n_launch, 4),
                      "gflop_per_launch": round(gemm_flops / n_launch / 1e9, 2),
