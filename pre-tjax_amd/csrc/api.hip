@@ -11,6 +11,28 @@ int ptj_set_error(int code, const char* fmt, ...) {
     return code;
 }
 
+// Compute units of the current device, asked once per device and kept.  Grid sizes of persistent
+// and grid-stride kernels are multiples of it.  Without a device (planning calls on a machine that
+// has none) the MI355X's 256.
+int ptj_num_cus() {
+    constexpr int DEFAULT_CUS = 256, MAX_DEVICES = 64;
+    static int cached[MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        return DEFAULT_CUS;
+    }
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = DEFAULT_CUS;
+        }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 extern "C" {
 int ptj_version(void) { return 1; }
 const char* ptj_last_error(void) { return g_err; }

@@ -832,7 +832,7 @@ int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t
     PTJ_CHECK_ARG(B >= 1 && T >= 32 && T % 32 == 0 && T < (1 << 24), "attn_pack_mask: need B >= 1 and T a multiple of 32");
     const int64_t words = 2 * B * (T / 32) * T;
     int64_t blocks = (words + 255) / 256;
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (blocks > (int64_t)ptj_num_cus() * 16) blocks = (int64_t)ptj_num_cus() * 16;
     hipLaunchKernelGGL(attn_pack_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, mask, packed, (int)B,
                        (int)T);
     PTJ_CHECK_LAUNCH();

@@ -519,7 +519,8 @@ int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* cou
     float* row_loss = (float*)ws;
     hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows, count);
     PTJ_CHECK_LAUNCH();
-    const int grid = (int)(rows < 256 * 2 ? rows : 256 * 2);
+    const int64_t two_per_cu = 2 * (int64_t)ptj_num_cus();
+    const int grid = (int)(rows < two_per_cu ? rows : two_per_cu);
     const bool cached = (cols + VEC) <= (int64_t)CE_THREADS * ITERS * VEC;
     if (cached)
         hipLaunchKernelGGL((ce_row_kernel<T, ITERS, true>), dim3(grid), dim3(1024), 0, st, labels, (const T*)logits,
@@ -534,7 +535,7 @@ int ce_impl(const int64_t* labels, const void* logits, float* loss, int64_t* cou
     return PTJ_OK;
 }
 
-constexpr int CE_CS_GRID = 256;   // one workgroup per CU (its LDS landing area fills the CU)
+inline int ce_cs_grid() { return ptj_num_cus(); }   // one workgroup per CU (its LDS landing area fills the CU)
 inline int ce_cs_pcols(int64_t cols) { return (int)((cols + 8 + 7) / 8 * 8); }
 
 }  // namespace
@@ -545,7 +546,7 @@ size_t ptj_ce_workspace_bytes(int64_t rows) { return rows > 0 ? (size_t)rows * s
 
 size_t ptj_ce_colsum_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
-    return ((size_t)rows * sizeof(float) + 255) / 256 * 256 + (size_t)CE_CS_GRID * ce_cs_pcols(cols) * sizeof(float);
+    return ((size_t)rows * sizeof(float) + 255) / 256 * 256 + (size_t)ce_cs_grid() * ce_cs_pcols(cols) * sizeof(float);
 }
 
 int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
@@ -567,7 +568,7 @@ int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss
     float* row_loss = (float*)workspace;
     float* part = (float*)((char*)workspace + ((size_t)rows * sizeof(float) + 255) / 256 * 256);
     const int pcols = ce_cs_pcols(cols);
-    const int grid = (int)(rows < CE_CS_GRID ? rows : CE_CS_GRID);
+    const int grid = (int)(rows < ce_cs_grid() ? rows : ce_cs_grid());
     const int mis = (int)((reinterpret_cast<uintptr_t>(logits) & 15) / 2);
     hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows, count);
     PTJ_CHECK_LAUNCH();

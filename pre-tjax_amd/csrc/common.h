@@ -19,6 +19,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 // ---- host-side error plumbing -------------------------------------------------
 int ptj_set_error(int code, const char* fmt, ...);
+int ptj_num_cus();   // compute units of the current device (256 when no device can be asked)
 
 #define PTJ_CHECK_ARG(cond, ...)                                   \
     do {                                                           \

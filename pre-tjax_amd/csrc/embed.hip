@@ -130,7 +130,7 @@ int embed_fwd_impl(const void* wemb, const void* pos, const int64_t* tokens, voi
     const bool vok = dim % FV == 0 && ptj_aligned16(wemb) && ptj_aligned16(pos) && ptj_aligned16(out);
     const int64_t work = n * (vok ? dim / FV : dim);
     int64_t blocks = (work + 255) / 256;
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (blocks > (int64_t)ptj_num_cus() * 16) blocks = (int64_t)ptj_num_cus() * 16;
     if (vok)
         hipLaunchKernelGGL((embed_fwd_kernel<T, FV>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)wemb, (const T*)pos,
                            tokens, (T*)out, n, (int)dim, seq, vocab, scale, train, (uint64_t)seed);

@@ -95,27 +95,8 @@ constexpr int TM = PTJ_GEMM_TM, TN = 3;     // 32x32 MFMA tiles per wavefront (r
 constexpr int WROWS = TM * 32;              // C rows per wavefront
 constexpr int WAVES_N = 2;                  // (BM/WROWS) x 2 wavefronts, each WROWS rows x 96 columns
 constexpr int GEMM_THREADS = (BM / WROWS) * WAVES_N * 64;
-constexpr int DEFAULT_CUS = 256;        // MI355X; used only when no device can be queried (planning calls without a GPU)
 
-// Compute units of the current device (persistent grid: one workgroup per CU), asked once per
-// device and kept.
-int num_cus() {
-    static int cached[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
-        (void)hipGetLastError();
-        return DEFAULT_CUS;
-    }
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-            (void)hipGetLastError();
-            n = DEFAULT_CUS;
-        }
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
+inline int num_cus() { return ptj_num_cus(); }   // persistent grid: one workgroup per CU
 
 // threadIdx.x behind an opaque barrier: everything derived from it (LDS and global
 // offsets) is recomputed per call instead of being hoisted out of the persistent tile

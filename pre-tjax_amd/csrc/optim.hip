@@ -192,7 +192,7 @@ int ptj_adamw(float* p, float* m, float* v, const void* g, void* shadow, int64_t
     const float bc2 = (float)(1.0 / (1.0 - pow((double)beta2, (double)t)));
     const int64_t n4 = n / 4;
     int64_t blocks = (n4 + 255) / 256;
-    if (blocks > 256 * 8) blocks = 256 * 8;
+    if (blocks > (int64_t)ptj_num_cus() * 8) blocks = (int64_t)ptj_num_cus() * 8;
     if (blocks < 1) blocks = 1;
     hipStream_t st = (hipStream_t)stream;
 #define ADAMW_LAUNCH(G_, S_, HS_)                                                                                  \

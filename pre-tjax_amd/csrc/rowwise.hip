@@ -875,7 +875,7 @@ inline bool pick_row_cfg(int64_t cols, int full_vec, bool vec_ok, RowCfg* cfg) {
 inline int row_grid(int64_t rows, int tpr) {
     const int rpb = tpr == 64 ? 4 : 1;
     const int64_t need = (rows + rpb - 1) / rpb;
-    const int64_t cap = 256 * 8;  // 8 workgroups per CU on 256 CUs
+    const int64_t cap = (int64_t)ptj_num_cus() * 8;  // 8 workgroups per CU
     return (int)(need < cap ? need : cap);
 }
 
@@ -1073,7 +1073,7 @@ int log_softmax_bwd_impl(const void* dy, const void* x, void* dx, int64_t rows, 
 
 inline int flat_grid(int64_t nthreads_needed) {
     int64_t b = (nthreads_needed + 255) / 256;
-    const int64_t cap = 256 * 16;
+    const int64_t cap = (int64_t)ptj_num_cus() * 16;
     if (b > cap) b = cap;
     if (b < 1) b = 1;
     return (int)b;
