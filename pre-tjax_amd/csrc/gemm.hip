@@ -61,7 +61,7 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     }
     g.partial = (splits > 1 || g.tail_splits > 1) ? (float*)workspace : nullptr;
     // streamed tiles need whole, evenly many K panels (the two-step loop body) and vector-aligned outputs
-    g.stream = (splits == 1 && g.vec_out && k >= STAGES * bk && k % (STAGES * bk) == 0) ? 1 : 0;
+    g.stream = (splits == 1 && g.vec_out && k >= 2 * bk && k % bk == 0) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     return dtype == PTJ_F32 ? ptj_gemm_detail::launch_plain_f32(g, splits, st) : gemm_impl<bf16>(g, splits, st);
 }

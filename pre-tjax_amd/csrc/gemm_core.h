@@ -80,7 +80,7 @@ constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from
 // kt+2 are issued during step kt and have one step to arrive; with 3, panel kt+3 is requested
 // during step kt and has two.
 #ifndef PTJ_GEMM_STAGES
-#define PTJ_GEMM_STAGES 2
+#define PTJ_GEMM_STAGES 3
 #endif
 // 1: within a step, all global loads of the incoming panel are issued first and the LDS stores of
 // the staged panel last (a load then has a step and a half to arrive); 0: store and load of a
@@ -89,8 +89,13 @@ constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from
 #ifndef PTJ_GEMM_EARLY_LOADS
 #define PTJ_GEMM_EARLY_LOADS 0
 #endif
-constexpr int STAGES = PTJ_GEMM_STAGES;
-static_assert(STAGES == 2 || STAGES == 3, "two or three staging register sets");
+static_assert(PTJ_GEMM_STAGES == 2 || PTJ_GEMM_STAGES == 3, "two or three staging register sets");
+// per operand layout and element size: only 2-byte operands that are copied as they are leave registers for a third
+// set (a transposing load holds its panel twice while it permutes: 104-126 spilled registers with three sets;
+// 4-byte storage: 50)
+constexpr int stages_for(int amode, int bmode, int elt) {
+    return (amode == KMAJOR && bmode == KMAJOR && elt == 2) ? PTJ_GEMM_STAGES : 2;
+}
 constexpr int TM = PTJ_GEMM_TM, TN = 3;     // 32x32 MFMA tiles per wavefront (rows x columns)
 constexpr int WROWS = TM * 32;              // C rows per wavefront
 constexpr int WAVES_N = 2;                  // (BM/WROWS) x 2 wavefronts, each WROWS rows x 96 columns
@@ -191,6 +196,7 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
                                               int row0, int col0, int kbeg, int nk) {
     constexpr int BK = BKB / (int)sizeof(T);
     constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+    constexpr int STAGES = stages_for(AMODE, BMODE, (int)sizeof(T));
     static_assert(TN == 3, "the pipeline below is written for three MFMA tile columns per wavefront");
     if (nk <= 0) return;
     const int tid = fresh_tid();
@@ -614,6 +620,7 @@ template <typename T, int AMODE, int BMODE, bool CLAMP, bool MUL>
 __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict__ smem) {
     constexpr int BK = BKB / (int)sizeof(T);
     constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+    constexpr int STAGES = stages_for(AMODE, BMODE, (int)sizeof(T));
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     const int total = num_m * num_n;
     // work items: whole tiles, then (with a K-split last round) the K slices of its tiles
@@ -935,6 +942,15 @@ int pick_mode(const void* p, int64_t s_row, int64_t s_k) {
 template <typename T, bool MUL = false>
 int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     const int am = pick_mode<T>(g.a, g.a_row, g.a_k), bm = pick_mode<T>(g.b, g.b_row, g.b_k);
+    {
+        // the streamed loop takes K panels in groups of as many as there are staging sets
+        const int sg = stages_for(am, bm, (int)sizeof(T)), bk = BKB / (int)sizeof(T);
+        if (g.stream && !(g.k >= sg * bk && g.k % (sg * bk) == 0)) g.stream = 0;
+        if (sg != 2 && g.tail_splits > 1) {      // K slices of the last round come in pairs of panels
+            g.tail_first = 0; g.tail_splits = 1; g.tail_kps = 0;
+            if (splits == 1) g.partial = nullptr;
+        }
+    }
     const int num_m = (g.n + BM - 1) / BM, num_n = (g.m + BN - 1) / BN;
     int64_t work = (int64_t)num_m * num_n * splits;
     if (g.tail_splits > 1) work = g.tail_first + ((int64_t)num_m * num_n - g.tail_first) * g.tail_splits;

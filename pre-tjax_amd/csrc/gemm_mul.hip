@@ -93,7 +93,7 @@ int ptj_gemm_mul_colsum(const void* a, const void* b, const void* mul, void* c, 
         const int64_t v = 16 / elt;
         g.vec_out = (ptj_aligned16(c) && c_rs % v == 0 && ptj_aligned16(mul) && mul_rs % v == 0 && ptj_aligned16(workspace) &&
                      m % 4 == 0) ? 1 : 0;
-        g.stream = (g.vec_out && k >= STAGES * bk && k % (STAGES * bk) == 0) ? 1 : 0;
+        g.stream = (g.vec_out && k >= 2 * bk && k % bk == 0) ? 1 : 0;
         const bool vector_operands =
             dtype == PTJ_F32 ? (pick_mode<float>(a, g.a_row, g.a_k) != GENERIC && pick_mode<float>(b, g.b_row, g.b_k) != GENERIC)
                              : (pick_mode<bf16>(a, g.a_row, g.a_k) != GENERIC && pick_mode<bf16>(b, g.b_row, g.b_k) != GENERIC);
