@@ -11,7 +11,7 @@ train mode, AdamW (lr 6e-4, betas 0.9/0.95, wd 0.1).
   sequences (an oracle forward pass over the whole batch takes 30 s on 16 host cores and a
   full oracle training step 90 s: 200 of them would take five hours), so every checked point
   is an independent comparison of the weights the run has reached.  The curve is written to
-  gpurun_out/ when that directory exists.
+  the directory named by PTJ_TEST_OUTPUT_DIR when that is set.
 
 The oracle runs in fp32 here (its own error, 1e-6, is far below the bf16 bars; fp64 would
 double its memory: the [B,H,T,T] probabilities of 12 layers are kept for autograd)."""
@@ -148,8 +148,8 @@ def test_c5_loss_curve_200_steps_b16_t1024(lo, data):
         assert curve[0] > math.log(V) + 1.0 and abs(curve[-1] - math.log(V)) < 0.15
     else:
         assert curve[-1] < curve[0] - 3.0, (curve[0], curve[-1])
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
+    out_dir = os.environ.get("PTJ_TEST_OUTPUT_DIR", "")
+    if out_dir and os.path.isdir(out_dir):
         with open(os.path.join(out_dir, "loss_curve_c5_%s.json" % data), "w") as f:
             json.dump({"data": data, "steps": steps, "B": B, "T": T, "loss": curve,
                        "oracle_checks_first_%d_sequences" % SUB: [{"step": s, "hip": a, "oracle": b}
