@@ -31,7 +31,6 @@ from util import rel_l2
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 CFG = dict(V=50257, D=768, L=12, H=12, F=3072, T=1024)
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def say(msg):
