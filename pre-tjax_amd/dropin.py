@@ -14,7 +14,8 @@ import importlib
 # kernel wrappers and composites of model_triton.py that the HIP library replaces
 MODEL_NAMES = (
     "t_log_softmax_fwd_t", "t_log_softmax_bkwd2_t", "t_gelu_fwd_t", "t_gelu_bkwd2_t", "t_matmul_t",
-    "t_tlayer_ffn_fwd_t", "t_tlayer_ffn_bkwd2_t", "t_scaled_dot_prod_attn_fwd3_t", "t_scaled_dot_prod_attn_bkwd3_t",
+    "t_tlayer_ffn_fwd_t", "t_tlayer_ffn_bkwd2_t", "t_softmax_attn_fwd_t", "t_softmax_attn_bkwd2_t",
+    "t_scaled_dot_prod_attn_fwd3_t", "t_scaled_dot_prod_attn_bkwd3_t",
     "t_dropout_fwd_t", "t_dropout_bkwd2_t", "t_layernorm_fwd_t", "t_layernorm_bkwd2_p_t", "t_layernorm_bkwd2_x_t",
     "t_gpt2_tlayer_fwd3_t", "t_gpt2_tlayer_bkwd3_t", "t_gpt2_tlayers_fwd3_t", "t_gpt2_forward_with_acts_t",
     "t_gpt2_bkwd3_p_t",

@@ -17,8 +17,8 @@ from ._lib import check, dtype_code, lib, ptr, require_gpu, stream
 from .spec_torch import (t_dropout_bkwd2, t_dropout_fwd, t_gelu_bkwd2, t_gelu_fwd,  # noqa: F401
                          t_layernorm_bkwd2_p, t_layernorm_bkwd2_x, t_layernorm_fwd, t_linear_fwd,
                          t_log_softmax_bkwd2, t_log_softmax_fwd, t_proj_fwd, t_scaled_dot_prod_attn_bkwd3,
-                         t_scaled_dot_prod_attn_fwd, t_scaled_dot_prod_attn_fwd3, t_softmax_attn_fwd,
-                         t_tlayer_ffn_fwd)
+                         t_scaled_dot_prod_attn_fwd, t_scaled_dot_prod_attn_fwd3, t_softmax_attn_bkwd2,
+                         t_softmax_attn_fwd, t_tlayer_ffn_fwd)
 
 DROPOUT_RATE = 0.1  # baked into the kernels, as in the reference (model_torch_func.py:2)
 
@@ -352,10 +352,17 @@ def t_matmul_t(a: torch.Tensor, b: torch.Tensor):
 t_matmul = t_matmul_t
 
 
+def _is_gelu_marker(fn):
+    """The reference passes its own `t_gelu_fwd` function object as a marker for "tanh-GELU"
+    (model_triton.py:1259, :2184); after an attribute-level install that object is the
+    reference module's, not this package's twin, so the marker is recognised by name."""
+    return getattr(fn, "__name__", "") in ("t_gelu_fwd", "t_gelu_fwd_t")
+
+
 def t_tlayer_ffn_fwd_t(layer_params, x: torch.Tensor, activation_fn=t_gelu_fwd):
     """Two GEMM launches: bias+GELU epilogue, then bias (model_triton.py:1258-1313).
     `activation_fn` is the reference's marker argument: its torch GELU (`t_gelu_fwd`)."""
-    assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU epilogue exists"
+    assert _is_gelu_marker(activation_fn), "only the tanh-GELU epilogue exists"
     w1, b1, w2, b2 = layer_params
     shape = x.shape
     x2 = _rows2d(x)
@@ -370,7 +377,7 @@ def t_tlayer_ffn_bkwd2_t(dloss_dx, layer_params, x: torch.Tensor, activation_fn=
     derivative), then dW2, db2, d(mid) times that derivative with db1 from the same launch,
     dW1 and dx.
     Returns (dx shaped like x, (dW1, db1, dW2, db2))."""
-    assert activation_fn in (t_gelu_fwd, t_gelu_fwd_t), "only the tanh-GELU backward exists"
+    assert _is_gelu_marker(activation_fn), "only the tanh-GELU backward exists"
     w1, b1, w2, b2 = layer_params
     x2 = _rows2d(x)
     d2 = _rows2d(dloss_dx)
@@ -515,6 +522,28 @@ def t_scaled_dot_prod_attn_bkwd3_t(dloss_dx, acts, qkv: torch.Tensor, mask: torc
         return dq[..., :dh] * f, dk[..., :dh].contiguous(), dv[..., :dh].contiguous()
     return attn_bwd_t(_aligned_view(dloss_dx), _aligned_view(q), _aligned_view(k), _aligned_view(v), _aligned_view(o), ms,
                       ls, mask, train, p_gen_aux)
+
+
+def _masked_scores(q, k, mask):
+    s = torch.matmul(q, k.transpose(-2, -1)) * (1.0 / math.sqrt(q.shape[-1]))
+    return s.masked_fill(~mask.unsqueeze(1), -1e9)
+
+
+def t_softmax_attn_fwd_t(q, k, mask, train, p_gen_aux=None):
+    """Materialised dropped attention probabilities [B,H,T,T] (model_triton.py:519-526): the
+    row-wise kernels (log-softmax, dropout) on torch's batched q.k^T.  Not on the training path
+    (the flash kernels never form this tensor); kept because callers import the name."""
+    return t_dropout_fwd_t(torch.exp(t_log_softmax_fwd_t(_masked_scores(q, k, mask))), train, p_gen_aux)
+
+
+def t_softmax_attn_bkwd2_t(dloss_dx, q, k, mask, train, p_gen_aux=None):
+    """VJP of t_softmax_attn_fwd_t with respect to (q, k) (model_triton.py:579-606)."""
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    s = _masked_scores(q, k, mask)
+    p = torch.exp(t_log_softmax_fwd_t(s))
+    d = t_dropout_bkwd2_t(dloss_dx, p, train, p_gen_aux) * p
+    d = t_log_softmax_bkwd2_t(d, s).masked_fill(~mask.unsqueeze(1), 0.0)
+    return torch.matmul(d, k) * scale, torch.matmul(d.transpose(-2, -1), q) * scale
 
 
 # ----------------------------------------------------------------------------------

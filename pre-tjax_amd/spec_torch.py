@@ -96,6 +96,17 @@ def t_softmax_attn_fwd(q, k, mask, train, p_gen_aux=None):
     return t_dropout_fwd(torch.exp(t_log_softmax_fwd(s)), train, p_gen_aux)
 
 
+def t_softmax_attn_bkwd2(dloss_dx, q, k, mask, train, p_gen_aux=None):
+    """(dq, dk) of t_softmax_attn_fwd for an incoming gradient of the dropped probabilities."""
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    s = (q @ k.transpose(-2, -1)) * scale
+    s = torch.where(mask.unsqueeze(1), s, torch.full_like(s, -1e9))
+    p = torch.softmax(s, dim=-1)
+    ds = t_log_softmax_bkwd2(t_dropout_bkwd2(dloss_dx, p, train, p_gen_aux) * p, s)
+    ds = torch.where(mask.unsqueeze(1), ds, torch.zeros_like(ds))
+    return (ds @ k) * scale, (ds.transpose(-2, -1) @ q) * scale
+
+
 def t_scaled_dot_prod_attn_fwd(qkv, mask, train=True, p_gen_aux=None):
     q, k, v = torch.unbind(qkv, dim=2)
     return t_softmax_attn_fwd(q, k, mask, train, p_gen_aux) @ v

@@ -18,6 +18,8 @@ MODEL_TRITON = {
     "t_matmul_t": (373, ["a", "b"], []),
     "t_tlayer_ffn_fwd_t": (1258, ["layer_params", "x", "activation_fn"], []),
     "t_tlayer_ffn_bkwd2_t": (1410, ["dloss_dx", "layer_params", "x", "activation_fn"], []),
+    "t_softmax_attn_fwd_t": (519, ["q", "k", "mask", "train", "p_gen_aux"], ["p_gen_aux"]),
+    "t_softmax_attn_bkwd2_t": (579, ["dloss_dx", "q", "k", "mask", "train", "p_gen_aux"], ["p_gen_aux"]),
     "t_scaled_dot_prod_attn_fwd3_t": (706, ["qkv", "mask", "train", "p_gen_aux"], ["train", "p_gen_aux"]),
     "t_scaled_dot_prod_attn_bkwd3_t": (951, ["dloss_dx", "acts", "qkv", "mask", "train", "p_gen_aux"],
                                        ["train", "p_gen_aux"]),
@@ -41,6 +43,7 @@ MODEL_TRITON = {
     "t_linear_fwd": (306, ["layer_params", "x"], []),
     "t_proj_fwd": (436, ["layer_params", "x"], []),
     "t_softmax_attn_fwd": (510, ["q", "k", "mask", "train", "p_gen_aux"], ["p_gen_aux"]),
+    "t_softmax_attn_bkwd2": (550, ["dloss_dx", "q", "k", "mask", "train", "p_gen_aux"], ["p_gen_aux"]),
     "t_scaled_dot_prod_attn_fwd": (608, ["qkv", "mask", "train", "p_gen_aux"], ["train", "p_gen_aux"]),
     "t_scaled_dot_prod_attn_fwd3": (756, ["qkv", "mask", "train", "p_gen_aux"], ["train", "p_gen_aux"]),
     "t_scaled_dot_prod_attn_bkwd3": (801, ["dloss_dx", "acts", "qkv", "mask", "train", "p_gen_aux"],
@@ -197,3 +200,42 @@ def test_install_patches_the_reference_modules_by_attribute(pkg):
         assert name in MODEL_TRITON, name
     for name in dropin.LOSS_NAMES:
         assert name in LOSS_AND_OPTIMIZER, name
+
+
+def test_ffn_wrappers_accept_the_reference_modules_own_gelu_marker(pkg):
+    """After an attribute-level install the callers pass THEIR module's `t_gelu_fwd` object
+    (model_triton.py:2184, tests/test_t_tlayer_ffn_fwd.py:21), which is not this package's twin:
+    the marker is recognised by name.  On CPU tensors the call then gets past the marker check
+    and stops at the no-fallback guard; anything that is not the GELU marker is refused."""
+    import importlib
+    dropin = importlib.import_module("pre-tjax_amd.dropin")
+    mt = importlib.import_module("pre-tjax_amd.model_triton")
+    lib = importlib.import_module("pre-tjax_amd._lib")
+    ref_mt = types.ModuleType("model_triton")
+
+    def t_gelu_fwd(x):                      # a distinct object with the reference's name
+        return x
+
+    ref_mt.t_gelu_fwd = t_gelu_fwd
+    dropin.install(ref_mt)
+    assert ref_mt.t_gelu_fwd is t_gelu_fwd and ref_mt.t_gelu_fwd is not mt.t_gelu_fwd
+    params = (torch.zeros(8, 4), torch.zeros(8), torch.zeros(4, 8), torch.zeros(4))
+    x = torch.zeros(2, 4)
+    for call in (lambda f: ref_mt.t_tlayer_ffn_fwd_t(params, x, f),
+                 lambda f: ref_mt.t_tlayer_ffn_bkwd2_t(x, params, x, f)):
+        with pytest.raises(lib.PtjError):
+            call(ref_mt.t_gelu_fwd)
+        with pytest.raises(AssertionError):
+            call(torch.relu)
+
+
+def test_softmax_attn_twin_backward_is_the_vjp_of_its_forward(mt):
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(2, 3, 5, 4, generator=g, dtype=torch.float64)
+    k = torch.randn(2, 3, 5, 4, generator=g, dtype=torch.float64)
+    mask = torch.tril(torch.ones(5, 5, dtype=torch.bool)).expand(2, 5, 5)
+    d = torch.randn(2, 3, 5, 5, generator=g, dtype=torch.float64)
+    qr, kr = q.clone().requires_grad_(True), k.clone().requires_grad_(True)
+    wq, wk = torch.autograd.grad(mt.t_softmax_attn_fwd(qr, kr, mask, False), (qr, kr), d)
+    gq, gk = mt.t_softmax_attn_bkwd2(d, q, k, mask, False)
+    assert torch.allclose(gq, wq, atol=1e-12) and torch.allclose(gk, wk, atol=1e-12)

@@ -41,3 +41,14 @@ def assert_close(got, want64, dtype, rtol=None, atol=None, what=""):
 def rel_l2(got, want64):
     g = f64(got)
     return ((g - want64).norm() / want64.norm().clamp_min(1e-30)).item()
+
+
+GEMM_ACC = 1e-5       # fp32 accumulation error of a product, relative to sum_k |a_ik b_kj|
+OUT_BF16 = 2.0 ** -8  # rounding of a result to bf16 (2^-9) with a factor two of slack, relative to the value
+
+
+def gemm_bound(want64, scale64, dtype, factor=1.0):
+    """Element-wise error bound of a matrix product with fp32 accumulation stored as `dtype`:
+    `scale64` = |a| @ |b| (+ |bias|), `want64` the exact result."""
+    out = OUT_BF16 if dtype == torch.bfloat16 else 0.0
+    return factor * GEMM_ACC * scale64 + out * want64.abs() + (1e-6 if dtype == torch.bfloat16 else 1e-30)
