@@ -284,15 +284,23 @@ int ptj_adamw_multi(int64_t count, float* const* p, float* const* m, float* cons
  * (model_triton.py:616-754).  ms/ls are contiguous [B*H, T].  Requires dh == 64, T % 64 == 0, 16-byte aligned
  * pointers and strides that are multiples of 16 bytes.  A non-NULL mask is applied
  * as (mask AND key <= query): masks must be sub-masks of the causal mask, as the
- * training path produces them.  `workspace` is needed when train != 0 only
- * (ptj_attn_workspace_bytes(B, H, T) bytes; the dropout keep bits live there). */
+ * training path produces them.  A query without any visible key (a padding row) gets an
+ * all-zero output row and the statistics (ms, ls) = (-1e9, 0), and the backward passes no
+ * gradient through it; the reference's kernel averages V over the keys of the tiles it
+ * happens to visit there (model_triton.py:678-682), its torch twin over all T keys -- such
+ * rows carry label 0 and are ignored by the loss.  `workspace` is needed when train != 0
+ * only (ptj_attn_workspace_bytes(B, H, T) bytes; the dropout keep bits live there). */
 size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T);
 
 /* Packs a uint8 [B, T, T] mask (nonzero = visible; contiguous) for the attention kernels:
  * one bit per (query, key), stored twice -- as words of 32 queries per key and as words of
  * 32 keys per query -- so that a wavefront fetches the mask of a 32x32 score tile with
- * scalar loads and applies it with lane-mask selects.  `packed` holds
- * ptj_attn_packed_mask_bytes(B, T) bytes (a quarter of the byte mask).  T % 32 == 0.
+ * scalar loads and applies it with lane-mask selects -- followed by one class word per
+ * 32x32 tile of (mask AND causal), in both index orders: hidden / mixed / equal to the causal
+ * pattern.  The kernels skip hidden tiles, read mask words only for mixed ones and mask by
+ * index elsewhere, so a plain lower-triangular mask tensor runs at the speed of mask = NULL.
+ * `packed` holds ptj_attn_packed_mask_bytes(B, T) bytes (about a quarter of the byte mask).
+ * T % 32 == 0.
  * The reference passes the bool mask itself to its kernels (model_triton.py:637, 672). */
 size_t ptj_attn_packed_mask_bytes(int64_t B, int64_t T);
 int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t T, void* stream);

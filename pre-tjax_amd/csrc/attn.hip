@@ -16,7 +16,16 @@
 //
 // Softmax is evaluated in base 2 (scores pre-multiplied by log2(e)/sqrt(dh)); the saved
 // statistics `ms` are converted back to natural units.  Masked scores take the
-// reference's fill value -1e9 (not -inf), including its behaviour on fully masked rows.
+// reference's fill value -1e9 (not -inf); the running maximum starts above it, so a masked
+// element contributes exactly 0.  A row without any visible key therefore has sum-exp 0: its
+// output row is 0, its saved statistics are (ms, ls) = (-1e9, 0), and the backward gives it
+// (and takes from it) no gradient.
+//
+// An explicit mask arrives bit-packed in both orientations together with one class per 32x32
+// tile of (mask AND causal): hidden everywhere / mixed / equal to the causal pattern.  Hidden
+// tiles are skipped, tiles equal to the causal pattern run the index-masked code, and only
+// mixed tiles read their mask words -- a plain lower-triangular tensor costs what mask = NULL
+// costs, and packed documents cost what they attend to.
 //
 // Dropout on the probabilities: element (q, k) of batch-head g is kept iff
 // philox(seed + g, q + k) passes the threshold -- the offset depends on q + k only, so
@@ -55,6 +64,7 @@ struct AttnArgs {
     // nullptr = causal by index; else the mask bit-packed in both orientations (ptj_attn_pack_mask):
     //   words [0, B*T/32*T):   word (b, q/32, k) holds M[b, 32*(q/32) + r, k] in bit r   (lane = query)
     //   then the same amount:  word (b, k/32, q) holds M[b, q, 32*(k/32) + r] in bit r   (lane = key)
+    //   then B*(T/32)^2 words:  class of tile (b, q/32, k/32), then the same indexed (b, k/32, q/32)
     const uint32_t* mask;
     float *ms, *ls;               // [BH, T]
     float* delta;                 // [BH, T] rowsum(dO * O)  (backward: written by the dQ pass, read by the dK/dV pass)
@@ -281,34 +291,67 @@ __global__ __launch_bounds__(256) void attn_pack_mask_kernel(const uint8_t* __re
     }
 }
 
+// Class of every 32x32 tile of (mask AND causal), from the packed words of orientation 0:
+//   TILE_CAUSAL  the tile equals the causal pattern (also every tile above the diagonal, where
+//                both are empty): index masking alone is exact
+//   TILE_HIDDEN  no element visible
+//   TILE_MIXED   anything else: the mask words are needed
+// written twice: cq[(b, q/32, k/32)] and ck[(b, k/32, q/32)].
+enum { TILE_HIDDEN = 0, TILE_MIXED = 1, TILE_CAUSAL = 2 };
+__global__ __launch_bounds__(256) void attn_mask_classes_kernel(const uint32_t* __restrict__ packed,
+                                                                 uint32_t* __restrict__ cq, uint32_t* __restrict__ ck,
+                                                                 int B, int T) {
+    const int G = T >> 5;
+    const int64_t total = (int64_t)B * G * G;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int kg = (int)(i % G), qg = (int)((i / G) % G);
+        const int64_t b = i / ((int64_t)G * G);
+        const uint32_t* w = packed + (b * G + qg) * (int64_t)T + 32 * kg;
+        bool any = false, same = true;
+        for (int c = 0; c < 32; ++c) {
+            const int d = 32 * kg + c - 32 * qg;   // query bit r is causally visible iff r >= d
+            const uint32_t cw = d <= 0 ? 0xffffffffu : (d >= 32 ? 0u : (0xffffffffu << d));
+            const uint32_t eff = w[c] & cw;
+            any |= eff != 0;
+            same &= eff == cw;
+        }
+        const uint32_t cls = same ? TILE_CAUSAL : (any ? TILE_MIXED : TILE_HIDDEN);
+        cq[i] = cls;
+        ck[(b * G + kg) * (int64_t)G + qg] = cls;
+    }
+}
+// classes of the two 32-wide halves of tile step `t` in the class row at `row` (wave-uniform)
+struct TileClasses { uint32_t c0, c1; };
+__device__ __forceinline__ TileClasses load_classes(const uint32_t* __restrict__ row, int t) {
+    TileClasses c;
+    c.c0 = row[2 * t];
+    c.c1 = row[2 * t + 1];
+    return c;
+}
+
 // ---- element-wise pieces (VALU budget: a wave64 VALU op costs 4 cycles, v_exp 16, and one
 //      K tile gives each lane 32 score elements against 16 MFMAs = 512 cycles; every
 //      instruction per element counts, so masks and dropout are compiled in only where used)
 constexpr float NEG_RAW = -8e9f;          // masked raw score: NEG_RAW * (1/sqrt(64)) = -1e9
 constexpr float RESCALE_SLACK = 8.0f;     // forward: the reference point of the exponentials may lag the row maximum by 2^8
-constexpr float MASKED_BELOW = -1e8f;     // log2-domain row max below this = fully masked row
+constexpr float M_START = -1e8f;          // log2-domain start of the running maximum: above every masked score
+                                          // (-1.44e9), below every real one, so exp2(masked - m) is exactly 0
 
-// Causal / explicit-mask visibility of the lane's 16 elements of sub-tile j written into
-// the raw scores (invisible -> NEG_RAW) and returned as a bit per element.
+// Causal visibility of the lane's 16 elements of a sub-tile written into the raw scores
+// (invisible -> NEG_RAW).
 //   pos0 = (lane's own index) - (first index of the sub-tile along registers) - 4*lg
 //   element i = 4a+b sits at register offset 8a+b: visible iff 8a+b <= pos0 (causal part).
 template <bool LANE_IS_QUERY>
-__device__ __forceinline__ uint32_t apply_causal(f32x16& s, int pos0) {
-    uint32_t bits = 0;
+__device__ __forceinline__ void apply_causal(f32x16& s, int pos0) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int off = (i >> 2) * 8 + (i & 3);
         // lane = query: key offset must be <= query;  lane = key: query offset must be >= key
         const bool ok = LANE_IS_QUERY ? (off <= pos0) : (off >= pos0);
         s[i] = ok ? s[i] : NEG_RAW;
-        bits |= ok ? (1u << i) : 0u;
     }
-    return bits;
 }
 
-__device__ __forceinline__ float and_bits(float v, int32_t m) { return __int_as_float(__float_as_int(v) & m); }
-// all-ones / all-zeros from bit `pos` of w
-__device__ __forceinline__ int32_t bit_mask(uint32_t w, int pos) { return __builtin_amdgcn_sbfe((int32_t)w, pos, 1); }
 
 // ---- forward -------------------------------------------------------------------------
 // grid (B*H, ceil(T/128)); wave w owns queries q0 + 32w .. +31; K/V tiles of 64 keys.
@@ -363,7 +406,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
     __syncthreads();
 
     const float sc = a.scale * LOG2E;
-    float m_run = NEG_RAW * sc, m_true = NEG_RAW * sc, l_run = 0.f;
+    float m_run = M_START, m_true = M_START, l_run = 0.f;
     f32x16 o[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -372,15 +415,26 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
 
     KeepWords kw_next;
     if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u);
+    // tile classes of the wave's 32 queries against every 32-key group (explicit mask only)
+    const uint32_t* __restrict__ crow = nullptr;
+    TileClasses tc_next = {TILE_CAUSAL, TILE_CAUSAL};
+    if constexpr (HAS_MASK) {
+        const int G = a.T >> 5;
+        crow = a.mask + 2 * (int64_t)a.B * G * a.T + ((int64_t)bidx * G + (qw0u >> 5)) * G;
+        tc_next = load_classes(crow, 0);
+    }
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
         FWD_FETCH(kt + 1 < nkt ? kt + 1 : kt)
-        // keep bits of this tile were requested one step ago; request the next tile's now
+        // keep bits and classes of this tile were requested one step ago; request the next tile's now
         const KeepWords kw = kw_next;
         if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u + (kt + 1) * 64);
+        const TileClasses tc = tc_next;
+        if constexpr (HAS_MASK) tc_next = load_classes(crow, kt + 1 < nkt ? kt + 1 : kt);
         __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
-        if (key0 <= qw0 + 31) {   // some key of this tile is visible to some query of the wave
+        // some key of this tile is visible to some query of the wave
+        if (key0 <= qw0 + 31 && (!HAS_MASK || (tc.c0 | tc.c1) != TILE_HIDDEN)) {
             const char* kp = smem + st * STAGE;
             const char* vp = kp + X::NP * PANEL;
             f32x16 s[2];
@@ -395,10 +449,12 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
                 for (int j = 0; j < 2; ++j) apply_causal<true>(s[j], query - key0 - j * 32 - lg * 4);
             }
             if constexpr (HAS_MASK) {
-                // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads)
+                // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads), read
+                // only for a half whose tile is not already described by the causal pattern
                 const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + key0;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
+                    if ((j == 0 ? tc.c0 : tc.c1) == TILE_CAUSAL) continue;
                     uint32_t w[32];
 #pragma unroll
                     for (int t = 0; t < 32; ++t) w[t] = mw[j * 32 + t];
@@ -453,12 +509,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_fwd_
 #undef FWD_STASH
 
     if (query < a.T) {
-        const float f = (TRAIN ? 1.0f : 0.9f) / l_run;
+        // l_run = 0: no key of the row is visible (a row with a visible key has l_run >= 1)
+        const bool empty = l_run == 0.f;
+        const float f = empty ? 0.f : (TRAIN ? 1.0f : 0.9f) / l_run;
         store_rows<T>((T*)a.out0 + bidx * a.out0_bs + hidx * a.out0_hs + (int64_t)query * a.out0_rs, o, f, lg);
         if (lg == 0) {
             // statistics relative to the true row maximum: sum exp(s - m_true) = l_run 2^(m_run - m_true)
-            a.ms[(int64_t)bh * a.T + query] = m_true < MASKED_BELOW ? NEG_NAT : m_true * LN2;
-            a.ls[(int64_t)bh * a.T + query] = l_run * fast_exp2(m_run - m_true);
+            a.ms[(int64_t)bh * a.T + query] = empty ? NEG_NAT : m_true * LN2;
+            a.ls[(int64_t)bh * a.T + query] = empty ? 0.f : l_run * fast_exp2(m_run - m_true);
         }
     }
 }
@@ -494,10 +552,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     TileLoader<T, KMAJOR, 64, ATT_THREADS> lq[X::NP], ld[X::NP];
     TileLoader<T, MNMAJOR, 64, ATT_THREADS, false, true> lqt[X::NP], ldt[X::NP];
     float st_m = 0.f, st_l = 1.f, st_d = 0.f;
-    // 2-byte storage without an explicit mask: 1/l goes into the exponent (p = 2^(s - m - log2 l)),
-    // one multiplication less per element.  Not with a mask: a fully masked row has m = -1e9,
-    // which would absorb log2 l.
-    constexpr bool FOLD_L = sizeof(T) == 2 && !HAS_MASK;
+    // 2-byte storage: 1/l goes into the exponent (p = 2^(s - m - log2 l)), one multiplication less
+    // per element.  A row without a visible key (saved l = 0) gets m = 0 and 1/l = 0 instead: all
+    // of its scores are masked (-1.44e9 in the exponent), so its p is exactly 0.
+    constexpr bool FOLD_L = sizeof(T) == 2;
     const int64_t stat0 = (int64_t)bh * a.T + (tid & 63);
 #define KV_FETCH(QT)                                                                   \
     {                                                                                  \
@@ -522,8 +580,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
             ldt[p].store(base__ + (3 * X::NP + p) * PANEL, tid);                       \
         }                                                                              \
         if (tid < 64) {                                                                \
-            sstat[ST][0][tid] = FOLD_L ? fmaf(st_m, LOG2E, __builtin_amdgcn_logf(st_l)) : st_m * LOG2E; \
-            sstat[ST][1][tid] = 1.0f / st_l;                                           \
+            const bool none__ = st_l == 0.f;                                           \
+            const float m2__ = FOLD_L ? fmaf(st_m, LOG2E, __builtin_amdgcn_logf(st_l)) : st_m * LOG2E; \
+            sstat[ST][0][tid] = none__ ? 0.f : m2__;                                   \
+            sstat[ST][1][tid] = none__ ? 0.f : 1.0f / st_l;                            \
             sstat[ST][2][tid] = st_d;                                                  \
         }                                                                              \
     }
@@ -546,11 +606,21 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
     const int kw0u = key0 + __builtin_amdgcn_readfirstlane(wave) * 32;
     KeepWords kw_next;
     if constexpr (TRAIN) kw_next = load_keep_words(kline, kw0u + qt0 * 64);
+    // tile classes of the wave's 32 keys against every 32-query group (explicit mask only)
+    const uint32_t* __restrict__ crow = nullptr;
+    TileClasses tc_next = {TILE_CAUSAL, TILE_CAUSAL};
+    if constexpr (HAS_MASK) {
+        const int G = a.T >> 5;
+        crow = a.mask + 2 * (int64_t)a.B * G * a.T + (int64_t)a.B * G * G + ((int64_t)bidx * G + (kw0u >> 5)) * G;
+        if (qt0 < nqt) tc_next = load_classes(crow, qt0);
+    }
     for (int qt = qt0; qt < nqt; ++qt) {
         const int st = (qt - qt0) & 1;
         KV_FETCH(qt + 1 < nqt ? qt + 1 : qt)
         const KeepWords kw = kw_next;   // requested one step ago
         if constexpr (TRAIN) kw_next = load_keep_words(kline, kw0u + (qt + 1) * 64);
+        const TileClasses tc = tc_next;
+        if constexpr (HAS_MASK) tc_next = load_classes(crow, qt + 1 < nqt ? qt + 1 : qt);
         __builtin_amdgcn_sched_barrier(0);
         const int q0 = qt * 64;
         if (q0 + 63 >= kw0) {   // some query of the tile sees some key of the wave
@@ -560,20 +630,21 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 if (q0 + j * 32 + 31 < kw0) continue;   // every query of this half precedes the wave's keys
+                const uint32_t cls = j == 0 ? tc.c0 : tc.c1;
+                if (HAS_MASK && cls == TILE_HIDDEN) continue;
                 f32x16 s, dp;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
                 rows_x_frags_one<T>(s, base, kf, j, lr, lg);                      // S  [query][key]
                 rows_x_frags_one<T>(dp, base + X::NP * PANEL, vf, j, lr, lg);     // dP [query][key]
 
-                uint32_t okbits = 0xffffu;
                 const bool diag = q0 + j * 32 < kw0 + 31;
-                if (diag) okbits = apply_causal<false>(s, key - q0 - j * 32 - lg * 4);
-                uint32_t mwords[32];
-                if constexpr (HAS_MASK) {
+                if (diag) apply_causal<false>(s, key - q0 - j * 32 - lg * 4);
+                if (HAS_MASK && cls != TILE_CAUSAL) {
                     // one word per query: the mask bits of the wave's 32 keys (wave-uniform loads)
                     const uint32_t* mw = a.mask + (int64_t)a.B * (a.T >> 5) * a.T +
                                          ((int64_t)bidx * (a.T >> 5) + (kw0u >> 5)) * a.T + q0 + j * 32;
+                    uint32_t mwords[32];
 #pragma unroll
                     for (int t = 0; t < 32; ++t) mwords[t] = mw[t];
 #pragma unroll
@@ -604,17 +675,9 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
                         }
                     }
                 }
-                // Causally hidden elements: without an explicit mask every query sees its own key,
-                // so the saved row statistics are finite and p (hence dS) is exactly 0 there;
-                // with a mask a fully masked row has p != 0 and dS is cleared explicitly.
-                if (HAS_MASK && diag) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
-                }
-                if constexpr (HAS_MASK) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[i] = mask_select(ds[i], 0.f, mask_lanes(mwords, i));
-                }
+                // Hidden elements (causal or masked) need no separate dS masking: their score is the
+                // fill value and the row's reference point is a real maximum (or 0 for a row without
+                // visible keys), so p, hence dS, is exactly 0 there.
                 tp_x_regs_one(dv, base + 3 * X::NP * PANEL, pd, j, lr, lg, T());  // dV^T += dO^T P
                 tp_x_regs_one(dk, base + 2 * X::NP * PANEL, ds, j, lr, lg, T());  // dK^T += Q^T dS
             }
@@ -658,9 +721,12 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 
     load_row_frags<T>(qf, Qb + (int64_t)qrow * a.q_rs, lg);
     load_row_frags<T>(dof, dOb + (int64_t)qrow * a.do_rs, lg);
     const int64_t si = (int64_t)bh * a.T + qrow;
-    // as in the dK/dV pass: 1/l folded into the exponent for 2-byte storage without a mask
-    constexpr bool FOLD_L = sizeof(T) == 2 && !HAS_MASK;
-    const float linv = 1.0f / a.ls[si];
+    // as in the dK/dV pass: 1/l folded into the exponent for 2-byte storage; a row without a
+    // visible key (saved l = 0) takes m = 0 and 1/l = 0, which makes its p exactly 0
+    constexpr bool FOLD_L = sizeof(T) == 2;
+    const float lsum = a.ls[si];
+    const bool none = lsum == 0.f;
+    const float linv = none ? 0.f : 1.0f / lsum;
     // delta = rowsum(dO * O) of the lane's query: each lane of the pair (lr, lg) holds one half
     // of the dO row already; the dK/dV pass (launched after this one) reads the stored values.
     float delta;
@@ -676,7 +742,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 
         delta = part + xor32(part);
         if (lg == 0 && query < a.T) a.delta[si] = delta;
     }
-    const float m2 = FOLD_L ? fmaf(a.ms[si], LOG2E, __builtin_amdgcn_logf(a.ls[si])) : a.ms[si] * LOG2E;
+    const float m2 = none ? 0.f : (FOLD_L ? fmaf(a.ms[si], LOG2E, __builtin_amdgcn_logf(lsum)) : a.ms[si] * LOG2E);
 
     int nkt = (q0 + 128) / 64;
     if (nkt > a.T / 64) nkt = a.T / 64;
@@ -711,11 +777,20 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 
     const int qw0u = q0 + __builtin_amdgcn_readfirstlane(wave) * 32;
     KeepWords kw_next;
     if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u);
+    const uint32_t* __restrict__ crow = nullptr;
+    TileClasses tc_next = {TILE_CAUSAL, TILE_CAUSAL};
+    if constexpr (HAS_MASK) {
+        const int G = a.T >> 5;
+        crow = a.mask + 2 * (int64_t)a.B * G * a.T + ((int64_t)bidx * G + (qw0u >> 5)) * G;
+        tc_next = load_classes(crow, 0);
+    }
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt & 1;
         DQ_FETCH(kt + 1 < nkt ? kt + 1 : kt)
         const KeepWords kw = kw_next;   // requested one step ago
         if constexpr (TRAIN) kw_next = load_keep_words(kline, qw0u + (kt + 1) * 64);
+        const TileClasses tc = tc_next;
+        if constexpr (HAS_MASK) tc_next = load_classes(crow, kt + 1 < nkt ? kt + 1 : kt);
         __builtin_amdgcn_sched_barrier(0);
         const int key0 = kt * 64;
         if (key0 <= qw0 + 31) {
@@ -726,19 +801,20 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 
             for (int j = 0; j < 2; ++j) {
                 const int kh0 = key0 + j * 32;
                 if (kh0 > qw0 + 31) continue;
+                const uint32_t cls = j == 0 ? tc.c0 : tc.c1;
+                if (HAS_MASK && cls == TILE_HIDDEN) continue;
                 f32x16 s, dp;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
                 rows_x_frags_one<T>(s, base, qf, j, lr, lg);                       // S^T  [key][query]
                 rows_x_frags_one<T>(dp, base + X::NP * PANEL, dof, j, lr, lg);     // dP^T [key][query]
 
-                uint32_t okbits = 0xffffu;
                 const bool masked = kh0 + 31 > qw0;
-                if (masked) okbits = apply_causal<true>(s, query - kh0 - lg * 4);
-                uint32_t mwords[32];
-                if constexpr (HAS_MASK) {
+                if (masked) apply_causal<true>(s, query - kh0 - lg * 4);
+                if (HAS_MASK && cls != TILE_CAUSAL) {
                     // one word per key: the mask bits of the wave's 32 queries (wave-uniform loads)
                     const uint32_t* mw = a.mask + ((int64_t)bidx * (a.T >> 5) + (qw0u >> 5)) * a.T + kh0;
+                    uint32_t mwords[32];
 #pragma unroll
                     for (int t = 0; t < 32; ++t) mwords[t] = mw[t];
 #pragma unroll
@@ -754,15 +830,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 
                     else
                         ds[i] = p * fmaf(dp[i], 0.9f, -delta);
                 }
-                // as in the dK/dV pass: only a masked launch can have p != 0 on hidden elements
-                if (HAS_MASK && masked) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[i] = and_bits(ds[i], bit_mask(okbits, i));
-                }
-                if constexpr (HAS_MASK) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) ds[i] = mask_select(ds[i], 0.f, mask_lanes(mwords, i));
-                }
+                // as in the dK/dV pass: p, hence dS, is exactly 0 on hidden elements
                 tp_x_regs_one(dq, base + 2 * X::NP * PANEL, ds, j, lr, lg, T());   // dQ^T += K^T dS^T
             }
         }
@@ -824,7 +892,8 @@ size_t ptj_attn_workspace_bytes(int64_t B, int64_t H, int64_t T) {
 
 size_t ptj_attn_packed_mask_bytes(int64_t B, int64_t T) {
     if (B < 1 || T < 32 || T % 32) return 0;
-    return (size_t)2 * B * (T / 32) * T * sizeof(uint32_t);
+    // the mask words in both orientations, then the tile classes in both index orders
+    return ((size_t)2 * B * (T / 32) * T + (size_t)2 * B * (T / 32) * (T / 32)) * sizeof(uint32_t);
 }
 
 int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t T, void* stream) {
@@ -835,6 +904,11 @@ int ptj_attn_pack_mask(const uint8_t* mask, uint32_t* packed, int64_t B, int64_t
     if (blocks > (int64_t)ptj_num_cus() * 16) blocks = (int64_t)ptj_num_cus() * 16;
     hipLaunchKernelGGL(attn_pack_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, mask, packed, (int)B,
                        (int)T);
+    PTJ_CHECK_LAUNCH();
+    const int64_t tiles = B * (T / 32) * (T / 32);
+    uint32_t* cq = packed + words;
+    hipLaunchKernelGGL(attn_mask_classes_kernel, dim3((unsigned)((tiles + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t*)packed, cq, cq + tiles, (int)B, (int)T);
     PTJ_CHECK_LAUNCH();
     return PTJ_OK;
 }

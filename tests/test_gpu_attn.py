@@ -97,6 +97,109 @@ def test_attn_padding_mask(mt, dtype, train):
     close(dv, wv, dtype, "dv")
 
 
+def _packed_documents_mask(B, T, seed):
+    """What the packing collator emits for a row of three documents and a padded tail:
+    lower triangular AND same document AND neither side padding.  Returns (mask [B,T,T] bool,
+    pad [B,T] bool: the queries without any visible key)."""
+    g = gen(seed)
+    doc = torch.zeros(B, T, dtype=torch.int64)
+    for b in range(B):
+        cuts = sorted(torch.randint(1, T - 40, (2,), generator=g).tolist())
+        end = int(torch.randint(T - 39, T - 3, (1,), generator=g))        # a padded tail of 4..39 positions
+        doc[b, :cuts[0]] = 1
+        doc[b, cuts[0]:cuts[1]] = 2
+        doc[b, cuts[1]:end] = 3                                            # 0 = padding
+    real = doc != 0
+    same = doc.unsqueeze(2) == doc.unsqueeze(1)
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool)) & same & real.unsqueeze(2) & real.unsqueeze(1)
+    return mask, ~real
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("train", [False, True])
+def test_attn_three_packed_documents_per_row(mt, dtype, train):
+    """Three packed documents and a padded tail per row at T = 512: hidden tiles (a later
+    document against an earlier one) are skipped, tiles inside a document run the index path,
+    tiles that straddle a document boundary or the padding read their mask words.  Rows with a
+    visible key against the oracle; padding queries (no visible key at all) give zero output
+    rows, statistics (-1e9, 0) and neither receive nor pass on gradient, so the oracle's
+    gradients are taken with dO zeroed on those rows."""
+    B, H, T, seed = 2, 3, 512, 515
+    qkv, dO, _ = make(B, H, T, dtype, seed=41)
+    mask, pad = _packed_documents_mask(B, T, 17)
+    assert pad.any() and (mask.sum(-1) == 0).equal(pad)
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), train, seed)
+    want_o = ops.scaled_dot_prod_attn_fwd(f64(qkv), mask, train, seed)
+    live = (~pad).view(B, 1, T, 1)
+    close(o * live.to(DEV), want_o * live, dtype, "O (rows with a visible key)")
+    padq = pad.view(B, 1, T).expand(B, H, T)
+    assert not o.cpu()[padq].any()                                          # exact zeros
+    assert (acts[0].cpu()[padq] == -1e9).all() and (acts[1].cpu()[padq] == 0).all()
+    ms, ls = ops.scaled_dot_prod_attn_stats(f64(qkv), mask)
+    st = torch.float32 if dtype == torch.float32 else dtype
+    close(torch.where(padq.to(DEV), 0, acts[0]), torch.where(padq, 0, ms), st, "ms")
+    close(torch.where(padq.to(DEV), 0, acts[1]), torch.where(padq, 0, ls), st, "ls")
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), train, seed)
+    wq, wk, wv = ops.scaled_dot_prod_attn_bkwd(f64(dO) * live, f64(qkv), mask, train, seed)
+    close(dq, wq, dtype, "dq")
+    close(dk, wk, dtype, "dk")
+    close(dv, wv, dtype, "dv")
+    assert not dq.cpu()[padq].any()
+    # keys that nobody sees (the padding) get no gradient either
+    assert not dk.cpu()[padq].any() and not dv.cpu()[padq].any()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_rows_without_visible_keys_closed_forms(mt, dtype):
+    """What the kernels do on rows the mask hides completely, next to rows with one visible key
+    (the reference's mask notebook, tests/test_t_scaled_dot_prod_attn_fwd_diff_masks.ipynb cells
+    1-3, compares such masks): a row whose only visible key is j returns 0.9 v_j (eval) whatever
+    the scores; a row with none returns 0 and has (ms, ls) = (-1e9, 0) -- also when every row of
+    its 32-query group is hidden (all tiles skipped) and when it sits in a group with live rows."""
+    B, H, T = 1, 2, 192
+    qkv, dO, _ = make(B, H, T, dtype, seed=5)
+    mask = torch.zeros(B, T, T, dtype=torch.bool)
+    idx = torch.arange(T)
+    one_key = (idx * 7) % (idx + 1)                       # some key <= query
+    mask[0, idx, one_key] = True
+    mask[0, 64:96] = False                                # a whole 32-query group without keys
+    mask[0, 130] = False                                  # single rows inside live groups
+    mask[0, 5] = False
+    hidden = mask.sum(-1) == 0
+    o, acts = mt.t_scaled_dot_prod_attn_fwd3_t(qkv.to(DEV), mask.to(DEV), False)
+    want = 0.9 * f64(qkv)[:, :, 2][:, :, one_key] * (~hidden).view(B, 1, T, 1)
+    close(o, want, dtype, "O")
+    hq = hidden.view(B, 1, T).expand(B, H, T)
+    assert not o.cpu()[hq].any()
+    assert (acts[0].cpu()[hq] == -1e9).all() and (acts[1].cpu()[hq] == 0).all()
+    assert (acts[1].cpu()[~hq] - 1).abs().max().item() < 1e-5   # one visible key: sum-exp = 1
+    dq, dk, dv = mt.t_scaled_dot_prod_attn_bkwd3_t(dO.to(DEV), acts, qkv.to(DEV), mask.to(DEV), False)
+    # one visible key per row: P is a one-hot row, so dS = 0 (dq = dk = 0 up to the rounding of the
+    # stored O inside rowsum(dO * O)) and dV_j = 0.9 * sum of dO_i over the live rows i whose key is j
+    want_dv = torch.zeros(B, H, T, 64, dtype=torch.float64)
+    want_dv.index_add_(2, one_key[~hidden[0]], 0.9 * f64(dO)[:, :, ~hidden[0]])
+    close(dv, want_dv, dtype, "dv")
+    tol = (1e-5 if dtype == torch.float32 else 2e-2) * want_dv.abs().max().item()
+    assert dq.abs().max().item() <= tol and dk.abs().max().item() <= tol
+    assert not dq.cpu()[hq].any()                         # rows without keys: exactly nothing
+
+
+@pytest.mark.parametrize("train", [False, True])
+def test_attn_lower_triangular_tensor_equals_mask_none_bitwise(mt, train):
+    """A plain lower-triangular mask tensor is classified tile by tile as the causal pattern and
+    runs the same index-masked code as mask=None: identical bits, forward and backward."""
+    B, H, T, seed = 2, 4, 512, 7
+    qkv, dO, mask = make(B, H, T, torch.bfloat16, seed=77)
+    qd, dd = qkv.to(DEV), dO.to(DEV)
+    o0, a0 = mt.t_scaled_dot_prod_attn_fwd3_t(qd, None, train, seed)
+    o1, a1 = mt.t_scaled_dot_prod_attn_fwd3_t(qd, mask.to(DEV), train, seed)
+    assert torch.equal(o0, o1) and torch.equal(a0[0], a1[0]) and torch.equal(a0[1], a1[1])
+    g0 = mt.t_scaled_dot_prod_attn_bkwd3_t(dd, a0, qd, None, train, seed)
+    g1 = mt.t_scaled_dot_prod_attn_bkwd3_t(dd, a1, qd, mask.to(DEV), train, seed)
+    for x, y in zip(g0, g1):
+        assert torch.equal(x, y)
+
+
 def test_attn_fresh_mask_tensor_every_call(mt):
     """The collator builds a new mask every batch: each call below gets a mask tensor that did
     not exist before, alternating between two contents, so that a freed mask's address is
