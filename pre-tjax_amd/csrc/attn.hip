@@ -699,7 +699,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 2 : 1) void attn_bwd_
 // Same geometry as the forward (lane = query, key tiles of 64).
 template <typename T, bool HAS_MASK, bool TRAIN>
 // (2-byte storage without an explicit mask fits three wavefronts per SIMD; the bound keeps it there)
-__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? (HAS_MASK ? 2 : 3) : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 3 : 1) void attn_bwd_dq_kernel(const AttnArgs a) {
     typedef AT<T> X;
     constexpr int STAGE = 3 * X::NP * PANEL;  // K, V, K^T
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];

@@ -930,6 +930,8 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const GemmArgs g)
     }
 }
 
+#include "gemm_direct.h"
+
 template <typename T>
 int pick_mode(const void* p, int64_t s_row, int64_t s_k) {
     constexpr int VEC = VecOf<T>::N;
@@ -956,6 +958,25 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
     if (g.tail_splits > 1) work = g.tail_first + ((int64_t)num_m * num_n - g.tail_first) * g.tail_splits;
     const int cus = num_cus();
     dim3 grid((unsigned)(work < cus ? work : cus)), block(GEMM_THREADS);
+    bool direct = false;
+    if constexpr (sizeof(T) == 2) {
+        // Operands that need a transpose on their way to the MFMAs (.t() views: the dX and dW products) take the
+        // loop with asynchronous copies and transposing LDS reads.  Two K-major operands stay on the register-staged
+        // loop, whose third staging set gives their loads two steps to arrive: inside a training step it is the
+        // faster of the two for them (4.67 against 4.90 ms over the step's 49 forward products), back to back
+        // in a loop it is the slower one.
+        direct = !(am == KMAJOR && bm == KMAJOR) && dg_eligible(g, am, bm);
+        if (direct) {
+#define DG_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_direct_kernel<AM, BMD, MUL>), grid, block, 0, st, g)
+            switch (am * 3 + bm) {
+                case 1: DG_LAUNCH(KMAJOR, MNMAJOR); break;
+                case 3: DG_LAUNCH(MNMAJOR, KMAJOR); break;
+                default: DG_LAUNCH(MNMAJOR, MNMAJOR); break;
+            }
+#undef DG_LAUNCH
+        }
+    }
+    if (!direct) {
 #define GEMM_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_kernel<T, AM, BMD, MUL>), grid, block, 0, st, g)
     if constexpr (MUL) {
         // the multiplying epilogue exists for vector-loadable operands only (the caller checks)
@@ -980,6 +1001,7 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
         }
     }
 #undef GEMM_LAUNCH
+    }
     PTJ_CHECK_LAUNCH();
     if (splits > 1) {
         const int64_t total = (int64_t)g.n * g.m;
