@@ -39,6 +39,7 @@ extern "C" {
 #define PTJ_EPI_BIAS 1           /* C = A.B + bias[m]                       */
 #define PTJ_EPI_BIAS_GELU 2      /* C = gelu(A.B + bias[m])                 */
 #define PTJ_EPI_BIAS_GELU_DERIV 3 /* the same C; c_pre = gelu'(A.B + bias[m]) */
+#define PTJ_EPI_ACCUMULATE 4     /* C = C + A.B (C is read, widened, and rounded once more) */
 
 int ptj_version(void);
 const char* ptj_last_error(void);
@@ -205,6 +206,21 @@ int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss
                           size_t workspace_bytes, int64_t rows, int64_t cols, int64_t logits_row_stride,
                           int64_t dlogits_row_stride, int dtype, void* stream);
 
+/* ptj_ce_fwd_bwd_colsum over the rows [row0, row0 + rows) of a problem of rows_total rows, for a caller
+ * that holds only a chunk of the logits at a time (LM head -> loss -> dX in row chunks: the
+ * reference materialises all [B, T, V] logits, model_triton.py:2538).  `labels` and `pred` are the
+ * whole arrays (rows_total entries), `logits` / `dlogits` point at the chunk's first row, the
+ * workspace is that of the whole problem (ptj_ce_colsum_workspace_bytes(rows_total, cols)) and must
+ * be left alone between the calls.  The call with row0 == 0 counts the labels != 0 of ALL rows
+ * (`count`), the call that reaches rows_total writes `loss` and `colsum`.  Chunks must be
+ * processed in row order with row0 a multiple of the device's CU count; then every addition
+ * happens in the order of the one-call form and the results are bit-equal to it. */
+int ptj_ce_fwd_bwd_colsum_rows(const int64_t* labels, const void* logits, float* loss, int64_t* count,
+                               void* dlogits, int64_t* pred, void* colsum, void* workspace,
+                               size_t workspace_bytes, int64_t rows_total, int64_t row0, int64_t rows,
+                               int64_t cols, int64_t logits_row_stride, int64_t dlogits_row_stride,
+                               int dtype, void* stream);
+
 /* ---- dense contraction --------------------------------------------------- */
 
 /* C[n,m] = sum_k A(n,k) * B(k,m) (+ bias[m]) (gelu) with fp32 accumulation on MFMA.
@@ -223,7 +239,11 @@ int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss
  * the activation the backward needs (the reference recomputes it, model_triton.py:1415-1418).
  * With PTJ_EPI_BIAS_GELU_DERIV `c_pre` (required) receives gelu'(A.B + bias) instead, taken from
  * the fp32 accumulators with the exponential the GELU needs anyway: what the backward multiplies
- * the incoming gradient by (t_gelu_bkwd2_k, model_triton.py:274-294). */
+ * the incoming gradient by (t_gelu_bkwd2_k, model_triton.py:274-294).
+ * PTJ_EPI_ACCUMULATE (no bias; 2-byte storage, 16-byte aligned operands with unit stride along one
+ * axis, k a multiple of 64, no K split: anything else is refused) starts the fp32 accumulators from
+ * the stored C: a weight gradient summed over row chunks of the batch (the reference forms it in one
+ * product over all rows, model_triton.py:423-428). */
 size_t ptj_gemm_workspace_bytes(int64_t n, int64_t m, int64_t k, int dtype);
 int ptj_gemm(const void* a, const void* b, void* c, const void* bias,
              int64_t n, int64_t m, int64_t k,

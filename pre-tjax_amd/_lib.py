@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libptj.so")
 
 PTJ_F32, PTJ_BF16 = 0, 1
-EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_BIAS_GELU_DERIV = 0, 1, 2, 3
+EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_BIAS_GELU_DERIV, EPI_ACCUMULATE = 0, 1, 2, 3, 4
 
 _c = ctypes
 _p, _i64, _int, _sz = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t
@@ -44,6 +44,7 @@ SIGNATURES = {
     "ptj_ce_fwd_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_ce_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_ce_fwd_bwd_colsum": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _int, _p]),
+    "ptj_ce_fwd_bwd_colsum_rows": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "ptj_gemm_mul_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_gemm_mul_colsum": (_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz, _int,

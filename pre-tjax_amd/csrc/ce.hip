@@ -330,7 +330,7 @@ __global__ __launch_bounds__(1024) void ce_row_colsum_kernel(const int64_t* __re
                                                               int64_t* __restrict__ pred,
                                                               const int64_t* __restrict__ count, int64_t rows, int cols,
                                                               int64_t xs, int64_t dxs, float* __restrict__ part,
-                                                              int pcols) {
+                                                              int pcols, int resume) {
     typedef bf16 T;
     constexpr int VEC = 8;
     __shared__ __attribute__((aligned(16))) char land[CE_THREADS * ITERS * 16];
@@ -342,11 +342,21 @@ __global__ __launch_bounds__(1024) void ce_row_colsum_kernel(const int64_t* __re
     // identical for every row
     const int mis = (int)((reinterpret_cast<uintptr_t>(logits) & 15) / sizeof(T));
     const int nvec = (cols + mis + VEC - 1) / VEC;
+    // resume: the rows given continue an earlier call's (same workgroup, same columns): the sums
+    // go on from the partial row that call left, so the additions keep the order of one call
     float acc[ITERS][VEC];
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it)
+    for (int it = 0; it < ITERS; ++it) {
+        const int vi = t + it * CE_THREADS;
+        f32x4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
+        if (resume && vi < nvec) {
+            const float* pr0 = part + (int64_t)blockIdx.x * pcols + vi * VEC;
+            lo4 = *reinterpret_cast<const f32x4*>(pr0);
+            hi4 = *reinterpret_cast<const f32x4*>(pr0 + 4);
+        }
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[it][j] = 0.f;
+        for (int j = 0; j < 4; ++j) { acc[it][j] = lo4[j]; acc[it][4 + j] = hi4[j]; }
+    }
     const int younger_stores = ce_exact_store_count<ITERS>(nvec, mis, cols, VEC);
     if ((int64_t)blockIdx.x < rows) ce_issue_row<T, ITERS>(logits + (int64_t)blockIdx.x * xs, cols, t, land);
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
@@ -549,44 +559,65 @@ size_t ptj_ce_colsum_workspace_bytes(int64_t rows, int64_t cols) {
     return ((size_t)rows * sizeof(float) + 255) / 256 * 256 + (size_t)ce_cs_grid() * ce_cs_pcols(cols) * sizeof(float);
 }
 
-int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
-                          int64_t* pred, void* colsum, void* workspace, size_t workspace_bytes, int64_t rows,
-                          int64_t cols, int64_t xs, int64_t dxs, int dtype, void* stream) {
+int ptj_ce_fwd_bwd_colsum_rows(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
+                               int64_t* pred, void* colsum, void* workspace, size_t workspace_bytes, int64_t rows_total,
+                               int64_t row0, int64_t rows, int64_t cols, int64_t xs, int64_t dxs, int dtype,
+                               void* stream) {
     PTJ_CHECK_ARG(labels && logits && loss && count && dlogits && colsum, "ce_fwd_bwd_colsum: null pointer");
     PTJ_CHECK_ARG(dtype == PTJ_BF16, "ce_fwd_bwd_colsum: 2-byte storage only (dtype %d)", dtype);
-    PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols + 8 <= (int64_t)CE_THREADS * CE_CS_MAX_ITERS * 8,
-                  "ce_fwd_bwd_colsum: bad shape %lld x %lld (at most %d columns)", (long long)rows, (long long)cols,
+    PTJ_CHECK_ARG(rows_total >= 1 && cols >= 1 && cols + 8 <= (int64_t)CE_THREADS * CE_CS_MAX_ITERS * 8,
+                  "ce_fwd_bwd_colsum: bad shape %lld x %lld (at most %d columns)", (long long)rows_total, (long long)cols,
                   CE_THREADS * CE_CS_MAX_ITERS * 8 - 8);
     PTJ_CHECK_ARG(xs >= cols && dxs >= cols && xs % 8 == 0 && dxs % 8 == 0,
                   "ce_fwd_bwd_colsum: row pitches must be multiples of 8 elements and at least cols");
     PTJ_CHECK_ARG(((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(dlogits)) & 15) == 0,
                   "ce_fwd_bwd_colsum: logits and dlogits must have equal 16-byte misalignment");
-    if (!workspace || workspace_bytes < ptj_ce_colsum_workspace_bytes(rows, cols))
+    if (!workspace || workspace_bytes < ptj_ce_colsum_workspace_bytes(rows_total, cols))
         return ptj_set_error(PTJ_ERR_WORKSPACE, "ce_fwd_bwd_colsum: workspace %zu < %zu bytes", workspace_bytes,
-                             ptj_ce_colsum_workspace_bytes(rows, cols));
+                             ptj_ce_colsum_workspace_bytes(rows_total, cols));
+    // one workgroup per CU over the WHOLE problem: workgroup w owns the rows w, w + grid, ... of it
+    const int grid = (int)(rows_total < ce_cs_grid() ? rows_total : ce_cs_grid());
+    PTJ_CHECK_ARG(rows >= 1 && row0 >= 0 && row0 + rows <= rows_total && row0 % grid == 0 &&
+                      (rows >= grid || row0 + rows == rows_total),
+                  "ce_fwd_bwd_colsum: rows [%lld, %lld) of %lld: chunks start at multiples of %d rows", (long long)row0,
+                  (long long)(row0 + rows), (long long)rows_total, grid);
     hipStream_t st = (hipStream_t)stream;
     float* row_loss = (float*)workspace;
-    float* part = (float*)((char*)workspace + ((size_t)rows * sizeof(float) + 255) / 256 * 256);
+    float* part = (float*)((char*)workspace + ((size_t)rows_total * sizeof(float) + 255) / 256 * 256);
     const int pcols = ce_cs_pcols(cols);
-    const int grid = (int)(rows < ce_cs_grid() ? rows : ce_cs_grid());
     const int mis = (int)((reinterpret_cast<uintptr_t>(logits) & 15) / 2);
-    hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows, count);
-    PTJ_CHECK_LAUNCH();
+    if (row0 == 0) {
+        hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows_total, count);
+        PTJ_CHECK_LAUNCH();
+    }
+    const int launch = (int)(rows < grid ? rows : grid);
+    const int resume = row0 > 0 ? 1 : 0;
+    int64_t* pred_rows = pred ? pred + row0 : nullptr;
     if (cols + 8 <= (int64_t)CE_THREADS * 4 * 8)
-        hipLaunchKernelGGL(ce_row_colsum_kernel<4>, dim3(grid), dim3(1024), 0, st, labels, (const bf16*)logits,
-                           (bf16*)dlogits, row_loss, pred, (const int64_t*)count, rows, (int)cols, xs, dxs, part, pcols);
+        hipLaunchKernelGGL(ce_row_colsum_kernel<4>, dim3(launch), dim3(1024), 0, st, labels + row0, (const bf16*)logits,
+                           (bf16*)dlogits, row_loss + row0, pred_rows, (const int64_t*)count, rows, (int)cols, xs, dxs,
+                           part, pcols, resume);
     else
-        hipLaunchKernelGGL(ce_row_colsum_kernel<CE_CS_MAX_ITERS>, dim3(grid), dim3(1024), 0, st, labels,
-                           (const bf16*)logits, (bf16*)dlogits, row_loss, pred, (const int64_t*)count, rows, (int)cols,
-                           xs, dxs, part, pcols);
+        hipLaunchKernelGGL(ce_row_colsum_kernel<CE_CS_MAX_ITERS>, dim3(launch), dim3(1024), 0, st, labels + row0,
+                           (const bf16*)logits, (bf16*)dlogits, row_loss + row0, pred_rows, (const int64_t*)count, rows,
+                           (int)cols, xs, dxs, part, pcols, resume);
     PTJ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)row_loss, rows,
-                       (const int64_t*)count, loss);
-    PTJ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(ce_colsum_reduce_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, st,
-                       (const float*)part, grid, pcols, mis, (int)cols, (bf16*)colsum);
-    PTJ_CHECK_LAUNCH();
+    if (row0 + rows == rows_total) {
+        hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)row_loss, rows_total,
+                           (const int64_t*)count, loss);
+        PTJ_CHECK_LAUNCH();
+        hipLaunchKernelGGL(ce_colsum_reduce_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, st,
+                           (const float*)part, grid, pcols, mis, (int)cols, (bf16*)colsum);
+        PTJ_CHECK_LAUNCH();
+    }
     return PTJ_OK;
+}
+
+int ptj_ce_fwd_bwd_colsum(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,
+                          int64_t* pred, void* colsum, void* workspace, size_t workspace_bytes, int64_t rows,
+                          int64_t cols, int64_t xs, int64_t dxs, int dtype, void* stream) {
+    return ptj_ce_fwd_bwd_colsum_rows(labels, logits, loss, count, dlogits, pred, colsum, workspace, workspace_bytes, rows,
+                                      0, rows, cols, xs, dxs, dtype, stream);
 }
 
 int ptj_ce_fwd_bwd(const int64_t* labels, const void* logits, float* loss, int64_t* count, void* dlogits,

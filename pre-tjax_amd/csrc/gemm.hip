@@ -18,9 +18,11 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
              void* workspace, size_t workspace_bytes, int dtype, void* stream) {
     PTJ_CHECK_ARG(n >= 0 && m >= 0 && k >= 0, "gemm: negative dimension");
     PTJ_CHECK_ARG(n < (1ll << 31) && m < (1ll << 31) && k < (1ll << 31), "gemm: dimension exceeds 31 bits");
-    PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_BIAS_GELU_DERIV, "gemm: unknown epilogue %d", epilogue);
+    PTJ_CHECK_ARG(epilogue >= PTJ_EPI_NONE && epilogue <= PTJ_EPI_ACCUMULATE, "gemm: unknown epilogue %d", epilogue);
     PTJ_CHECK_ARG(epilogue != PTJ_EPI_BIAS_GELU_DERIV || c_pre, "gemm: the derivative epilogue needs its second output");
-    PTJ_CHECK_ARG(epilogue == PTJ_EPI_NONE || bias, "gemm: epilogue %d needs a bias", epilogue);
+    PTJ_CHECK_ARG(epilogue == PTJ_EPI_NONE || epilogue == PTJ_EPI_ACCUMULATE || bias, "gemm: epilogue %d needs a bias", epilogue);
+    PTJ_CHECK_ARG(epilogue != PTJ_EPI_ACCUMULATE || (!bias && !c_pre && dtype == PTJ_BF16),
+                  "gemm: the accumulating epilogue takes no bias and no second output, 2-byte storage only");
     PTJ_CHECK_ARG(dtype == PTJ_F32 || dtype == PTJ_BF16, "gemm: unknown dtype %d", dtype);
     if (n == 0 || m == 0) return PTJ_OK;
     PTJ_CHECK_ARG(c && (k == 0 || (a && b)), "gemm: null pointer");
@@ -39,6 +41,7 @@ int ptj_gemm(const void* a, const void* b, void* c, const void* bias, int64_t n,
     g.c_aux_rs = c_pre_rs;
     g.epilogue = epilogue;
     g.mul = nullptr; g.mul_rs = 0; g.colpart = nullptr;
+    if (epilogue == PTJ_EPI_ACCUMULATE) workspace = nullptr;   // no K split: the partial sums would not see the stored C
     int splits = workspace ? choose_splits(n, m, k, elt, workspace_bytes) : 1;
     int64_t kps = k;
     if (splits > 1) {

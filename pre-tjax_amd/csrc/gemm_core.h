@@ -966,6 +966,10 @@ int gemm_impl(GemmArgs g, int splits, hipStream_t st) {
         // faster of the two for them (4.67 against 4.90 ms over the step's 49 forward products), back to back
         // in a loop it is the slower one.
         direct = !(am == KMAJOR && bm == KMAJOR) && dg_eligible(g, am, bm);
+        // only the loop with asynchronous copies starts its accumulators from the stored C
+        if (g.epilogue == PTJ_EPI_ACCUMULATE && !(direct && g.vec_out && splits == 1 && g.tail_splits <= 1))
+            return ptj_set_error(PTJ_ERR_INVALID, "gemm: the accumulating epilogue needs a transposed 16-byte aligned "
+                                 "operand layout, k a multiple of 64 and vector-aligned C");
         if (direct) {
 #define DG_LAUNCH(AM, BMD) hipLaunchKernelGGL((gemm_direct_kernel<AM, BMD, MUL>), grid, block, 0, st, g)
             switch (am * 3 + bm) {

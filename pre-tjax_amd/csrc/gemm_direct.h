@@ -199,6 +199,38 @@ __device__ __forceinline__ DgItem dg_item(const GemmArgs& g, int item, int num_m
     return d;
 }
 
+// PTJ_EPI_ACCUMULATE: the accumulators of the tile at (row0, col0) start from the stored C.  acc[tn][tm][i] of
+// lane (lr, lg) is C[row0 + wm*64 + tm*32 + lr][col0 + wn*96 + tn*32 + (i/4)*8 + lg*4 + i%4]: four consecutive
+// columns per load.  Elements outside C start from zero (their results are never stored).
+template <bool CLAMP>
+__device__ __forceinline__ void dg_load_c_tile(const GemmArgs& g, f32x16 (&acc)[TN][TM], int row0, int col0) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int r0 = row0 + (wave / WAVES_N) * WROWS + lr, c0 = col0 + (wave % WAVES_N) * 96 + lg * 4;
+    const bf16* C = (const bf16*)g.c;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int row = r0 + tm * 32, col = c0 + tn * 32 + q * 8;
+                Pack<bf16, 4> v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v.v[e] = from_f32<bf16>(0.f);
+                if (!CLAMP || (row < g.n && col + 4 <= g.m)) {
+                    v = *reinterpret_cast<const Pack<bf16, 4>*>(C + (int64_t)row * g.c_rs + col);
+                } else if (row < g.n) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < g.m) v.v[e] = C[(int64_t)row * g.c_rs + col + e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[tn][tm][q * 4 + e] = to_f32(v.v[e]);
+            }
+}
+
 template <int AMODE, int BMODE, bool CLAMP, bool MUL>
 __device__ __forceinline__ void gemm_direct(const GemmArgs& g, char* __restrict__ smem) {
     typedef bf16 T;
@@ -293,6 +325,9 @@ __device__ __forceinline__ void gemm_direct(const GemmArgs& g, char* __restrict_
             for (int j = 0; j < TM; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = to_f32(braw[i * 4 + (e >> 2)].v[e & 3]);
+        if constexpr (!MUL) {
+            if (g.epilogue == PTJ_EPI_ACCUMULATE) dg_load_c_tile<CLAMP>(g, acc, cur.row0, cur.col0);
+        }
         for (int kt = 0; kt < cur.nk; ++kt) {
             const uint32_t sa = pb * DG_A_BYTES, sb = pb * DG_B_BYTES;
             const uint32_t na = (pb ^ 1) * DG_A_BYTES, nb = (pb ^ 1) * DG_B_BYTES;

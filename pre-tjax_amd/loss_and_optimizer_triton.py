@@ -70,12 +70,70 @@ def accuracy_from_pred(y_labels, pred):
     return torch.nanmean(torch.where(y_labels != 0, hit, torch.full_like(hit, float("nan"))))
 
 
+LM_HEAD_CHUNK_ROWS = 8192   # rows of logits alive at a time in t_loss_bkwd3_t (0: all of them, one pass)
+
+
+def _lm_head_loss_in_row_chunks(params, h, y_out, chunk):
+    """LM head -> loss -> the head's three gradient products, `chunk` rows at a time: only
+    [chunk, V] logits exist at any moment (the reference materialises [B, T, V],
+    model_triton.py:2538, and a same-sized gradient, loss_and_optimizer_triton.py:176-197).
+    Per chunk: logits = h_c @ Wemb^T + bemb into one reused row-padded buffer, the loss pass
+    overwrites them with their gradient (continuing the loss sum, the argmax and the column sums of
+    the previous chunks), dh_c = dlogits_c @ Wemb, and dWemb += dlogits_c^T @ h_c (accumulating
+    epilogue: the stored sum is widened, added to and rounded once per chunk).
+    Returns (loss[1], count, pred [B,T], dh [N,D], dwemb [V,D], dbemb [V])."""
+    from .model_triton import _padded_logits, matmul_t
+    wemb, bemb = params[0]
+    V, D = wemb.shape
+    N = y_out.numel()
+    h2d = h.reshape(N, D)
+    labels = y_out.reshape(-1).to(torch.int64).contiguous()
+    dev = h.device
+    loss = torch.empty(1, dtype=torch.float32, device=dev)
+    count = torch.empty((), dtype=torch.int64, device=dev)
+    pred = torch.empty(N, dtype=torch.int64, device=dev)
+    dbemb = torch.empty(V, dtype=h.dtype, device=dev)
+    dh = torch.empty((N, D), dtype=h.dtype, device=dev)
+    dwemb = torch.empty((V, D), dtype=h.dtype, device=dev)
+    buf = _padded_logits(chunk, V, h.dtype, dev)
+    ws_bytes = lib().ptj_ce_colsum_workspace_bytes(N, V)
+    ws = _workspace(ws_bytes, dev, "ce")
+    for r0 in range(0, N, chunk):
+        rows = min(chunk, N - r0)
+        lg = buf[:rows]
+        matmul_t(h2d[r0:r0 + rows], wemb.t(), bemb, out=lg)
+        check(lib().ptj_ce_fwd_bwd_colsum_rows(ptr(labels), ptr(lg), ptr(loss), ptr(count), ptr(lg), ptr(pred), ptr(dbemb),
+                                               ptr(ws), ws_bytes, N, r0, rows, V, lg.stride(0), lg.stride(0),
+                                               dtype_code(lg), stream()), "ptj_ce_fwd_bwd_colsum_rows")
+        matmul_t(lg, wemb, out=dh[r0:r0 + rows])
+        matmul_t(lg.t(), h2d[r0:r0 + rows], out=dwemb, accumulate=r0 > 0)
+    return loss, count, pred.reshape(y_out.shape), dh, dwemb, dbemb
+
+
+def _chunked_head_applies(params, n_rows, chunk):
+    """Row chunks need the fused loss pass (2-byte logits, vocabulary within its register budget)
+    and chunk starts at multiples of the loss pass's workgroup count (one per CU)."""
+    wemb = params[0][0]
+    return (chunk > 0 and n_rows > chunk and wemb.dtype == torch.bfloat16 and wemb.shape[0] + 8 <= 1024 * 56
+            and chunk % 1024 == 0 and wemb.shape[1] % 64 == 0 and chunk % 64 == 0)
+
+
 def t_loss_bkwd3_t(params, y, y_mask, y_indices, train, p_gen_aux=None):
     """One forward+backward (reference: loss_and_optimizer_triton.py:279-289).
-    y int [B,T+1] -> (grads nest, (loss, acc, non-pad fraction))."""
-    from .model_triton import t_gpt2_bkwd3_p_t, t_gpt2_forward_with_acts_t
+    y int [B,T+1] -> (grads nest, (loss, acc, non-pad fraction)).  With more than
+    LM_HEAD_CHUNK_ROWS positions in 2-byte storage, the LM head, the loss and the head's gradient
+    products run in row chunks (see _lm_head_loss_in_row_chunks); otherwise in one pass over a
+    [B, T, V] logits buffer."""
+    from .model_triton import (gpt2_bkwd_below_head_t, t_gpt2_bkwd3_p_t, t_gpt2_forward_with_acts_t,
+                               t_gpt2_tlayers_fwd3_t)
     y_in = y[:, :-1]
     y_out = y[:, 1:]
+    if _chunked_head_applies(params, y_out.numel(), LM_HEAD_CHUNK_ROWS):
+        h, acts = t_gpt2_tlayers_fwd3_t(params, y_in, y_mask, y_indices, train, p_gen_aux)
+        loss_val, tokens_count, pred, dh, dwemb, dbemb = _lm_head_loss_in_row_chunks(params, h, y_out, LM_HEAD_CHUNK_ROWS)
+        grads = gpt2_bkwd_below_head_t(dh, dwemb, dbemb, [acts, h], params, y_in, y_mask, train, p_gen_aux)
+        acc = accuracy_from_pred(y_out, pred)
+        return grads, (loss_val, acc, tokens_count / y_out.numel())
     logits, acts = t_gpt2_forward_with_acts_t(params, y_in, y_mask, y_indices, train, p_gen_aux)
     # the bias gradient of the tied head (column sums of the loss gradient) comes out of the loss pass
     loss_val, tokens_count, dloss_dx, pred, dbemb = t_avg_cross_entropy_loss_bkwd3_t(y_out, logits, inplace=True,

@@ -285,23 +285,33 @@ def colsum_t(x: torch.Tensor):
 # ----------------------------------------------------------------------------------
 # GEMM  (reference: model_triton.py:373-398 t_matmul_t, :1258-1313 t_tlayer_ffn_fwd_t)
 # ----------------------------------------------------------------------------------
-def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, pre_out=None, deriv_out=None):
+def matmul_t(a: torch.Tensor, b: torch.Tensor, bias=None, gelu=False, out=None, pre_out=None, deriv_out=None,
+             accumulate=False):
     """``out[N,M] = a[N,K] @ b[K,M] (+ bias[M]) (tanh-GELU)`` on the MFMA GEMM kernel.
 
     `a` and `b` are 2-D tensors with arbitrary strides (``.t()`` views are consumed in
     place, never copied); `out`, if given, is a 2-D tensor with unit column stride
     (a column slice of a wider buffer is fine).  `pre_out` (with ``gelu=True``) also
     receives ``a @ b + bias`` before the activation; `deriv_out` (instead) receives the
-    GELU's derivative there, which is all the backward pass needs of it."""
+    GELU's derivative there, which is all the backward pass needs of it.  With
+    ``accumulate=True`` the product is added onto the given `out` (the accumulators start from
+    it): a weight gradient summed over row chunks."""
     require_gpu(a, b, bias, out)
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], (a.shape, b.shape)
     assert a.dtype == b.dtype
     N, K = a.shape
     M = b.shape[1]
     if out is None:
+        assert not accumulate, "accumulate needs the tensor to add onto"
         out = torch.empty((N, M), dtype=a.dtype, device=a.device)
     else:
         assert out.shape == (N, M) and out.dtype == a.dtype and (out.stride(1) == 1 or M == 1)
+    if accumulate:
+        assert bias is None and not gelu and pre_out is None and deriv_out is None
+        check(lib().ptj_gemm(ptr(a), ptr(b), ptr(out), None, N, M, K, a.stride(0), a.stride(1), b.stride(0),
+                             b.stride(1), out.stride(0), _lib.EPI_ACCUMULATE, None, 0, None, 0, dtype_code(a), stream()),
+              "ptj_gemm")
+        return out
     epi = _lib.EPI_NONE
     if bias is not None:
         assert bias.dtype == a.dtype and bias.numel() == M
@@ -757,6 +767,20 @@ def t_gpt2_bkwd3_p_t(dloss_dx, acts, params, y, y_mask, y_indices, train, p_gen_
         dbemb = colsum_t(dlog)
     dwemb = matmul_t(dlog.t(), h2d)                                     # [V,D]  LM-head weight grad
     dh = matmul_t(dlog, wemb)                                           # [N,D]
+    return gpt2_bkwd_below_head_t(dh, dwemb, dbemb, acts, params, y, y_mask, train, p_gen_aux)
+
+
+def gpt2_bkwd_below_head_t(dh, dwemb, dbemb, acts, params, y, y_mask, train, p_gen_aux=None):
+    """t_gpt2_bkwd3_p_t from the gradient of the final LayerNorm's output on (model_triton.py:2583-2593
+    after the LM head's own three products): `dh` [N,D] = dlogits @ Wemb, `dwemb` [V,D] = the head's
+    weight gradient (the embedding's is added onto it), `dbemb` [V] its bias gradient."""
+    L = len(params) - 3
+    if not train:
+        p_gen_aux = [0] * (1 + 3 * L)
+    (layer_acts, x_last), _ = acts
+    D = dh.shape[1]
+    B, T = y.shape
+    N = B * T
     # Every dropout backward acts on a gradient that a LayerNorm backward has just produced,
     # so each LayerNorm backward also writes the dropped copy its consumer needs: the final
     # norm for the last block's FFN dropout (seed 3L), block i's first norm for block i-1's

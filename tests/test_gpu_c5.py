@@ -80,7 +80,14 @@ def test_c5_one_step_b2_t1024_bf16_train_vs_oracle(lo):
     dparams = [[p.to(DEV) for p in grp] for grp in bf]
     for mask_as in ("none", "tensor"):
         dmask = mask.to(DEV) if mask_as == "tensor" else None
-        grads, (loss, acc, frac) = lo.t_loss_bkwd3_t(dparams, y.to(DEV), dmask, None, True, seeds)
+        # the 2048 positions fit one pass of the LM head; the tensor-mask run takes it in two row
+        # chunks instead, so that the chunked form of the head is held to the oracle as well
+        chunk_rows = lo.LM_HEAD_CHUNK_ROWS
+        lo.LM_HEAD_CHUNK_ROWS = 1024 if mask_as == "tensor" else chunk_rows
+        try:
+            grads, (loss, acc, frac) = lo.t_loss_bkwd3_t(dparams, y.to(DEV), dmask, None, True, seeds)
+        finally:
+            lo.LM_HEAD_CHUNK_ROWS = chunk_rows
         assert abs(loss.item() - wl.item()) <= 5e-3 * abs(wl.item()), (mask_as, loss.item(), wl.item())
         assert abs(frac.item() - wfrac.item()) < 1e-6
         worst, where = 0.0, None
