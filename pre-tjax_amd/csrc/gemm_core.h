@@ -69,34 +69,18 @@ int launch_plain_f32(const GemmArgs& g, int splits, hipStream_t st);   // gemm_f
 namespace {
 using ptj_gemm_detail::GemmArgs;
 
-#ifndef PTJ_GEMM_BM
-#define PTJ_GEMM_BM 256
-#endif
-constexpr int BM = PTJ_GEMM_BM, BN = 192;   // C tile (rows from A, columns from B)
-#ifndef PTJ_GEMM_TM
-#define PTJ_GEMM_TM 2
-#endif
+constexpr int BM = 256, BN = 192;   // C tile (rows from A, columns from B)
 // Register sets that stage operand panels between HBM and LDS: with 2, the loads of panel
 // kt+2 are issued during step kt and have one step to arrive; with 3, panel kt+3 is requested
 // during step kt and has two.
-#ifndef PTJ_GEMM_STAGES
-#define PTJ_GEMM_STAGES 3
-#endif
-// 1: within a step, all global loads of the incoming panel are issued first and the LDS stores of
-// the staged panel last (a load then has a step and a half to arrive); 0: store and load of a
-// slice side by side, spread over the step.  Measured on one box: 20.25 ms per training step with
-// 1, 19.62 ms with 0.
-#ifndef PTJ_GEMM_EARLY_LOADS
-#define PTJ_GEMM_EARLY_LOADS 0
-#endif
-static_assert(PTJ_GEMM_STAGES == 2 || PTJ_GEMM_STAGES == 3, "two or three staging register sets");
+constexpr int GEMM_MAX_STAGES = 3;
 // per operand layout and element size: only 2-byte operands that are copied as they are leave registers for a third
 // set (a transposing load holds its panel twice while it permutes: 104-126 spilled registers with three sets;
 // 4-byte storage: 50)
 constexpr int stages_for(int amode, int bmode, int elt) {
-    return (amode == KMAJOR && bmode == KMAJOR && elt == 2) ? PTJ_GEMM_STAGES : 2;
+    return (amode == KMAJOR && bmode == KMAJOR && elt == 2) ? GEMM_MAX_STAGES : 2;
 }
-constexpr int TM = PTJ_GEMM_TM, TN = 3;     // 32x32 MFMA tiles per wavefront (rows x columns)
+constexpr int TM = 2, TN = 3;               // 32x32 MFMA tiles per wavefront (rows x columns)
 constexpr int WROWS = TM * 32;              // C rows per wavefront
 constexpr int WAVES_N = 2;                  // (BM/WROWS) x 2 wavefronts, each WROWS rows x 96 columns
 constexpr int GEMM_THREADS = (BM / WROWS) * WAVES_N * 64;
@@ -233,36 +217,6 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
 #define ST_B(I, LWB, P) LWB.template store_slice<I, 3>(sB + ((P) ^ 1) * B_BYTES, tid)
 #define LD_A(I, LFA, KTF) LFA.template load_fast_slice<I, 4, CLAMP>(A, g.a_row, g.a_k, ROW_A(KTF), K0_OF(KTF), tid, g.n)
 #define LD_B(I, LFB, KTF) LFB.template load_fast_slice<I, 3, CLAMP>(B, g.b_row, g.b_k, ROW_B(KTF), K0_OF(KTF), tid, g.m)
-#if PTJ_GEMM_EARLY_LOADS
-    // The set that receives panel KTF was written to LDS during the previous step, so all of its
-    // loads can go out in the first third of the step; the set that holds panel kt+1 is stored in
-    // the last half.  A load then has about a step and a half to arrive before its store needs it.
-#define RF_STEP(P, LWA, LWB, LFA, LFB, KTF)                                                               \
-    do {                                                                                                  \
-        RD_A(P, 1, 1); SB();                                                                              \
-        MM(0, fb[0], 0); SB();                                                                            \
-        RD_B(fb[0], P, 1, 0); LD_A(0, LFA, KTF); LD_A(1, LFA, KTF); SB();                                 \
-        MM(1, fb[1], 0); SB();                                                                            \
-        RD_B(fb[1], P, 1, 1); LD_A(2, LFA, KTF); LD_A(3, LFA, KTF); SB();                                 \
-        MM(2, fb[2], 0); SB();                                                                            \
-        RD_B(fb[2], P, 1, 2); LD_B(0, LFB, KTF); LD_B(1, LFB, KTF); LD_B(2, LFB, KTF); SB();              \
-        RD_A(P, 2, 0); SB();                                                                              \
-        MM(0, fb[0], 1); SB();                                                                            \
-        RD_B(fb[0], P, 2, 0); ST_A(0, LWA, P); ST_A(1, LWA, P); SB();                                     \
-        MM(1, fb[1], 1); SB();                                                                            \
-        RD_B(fb[1], P, 2, 1); ST_A(2, LWA, P); ST_A(3, LWA, P); SB();                                     \
-        MM(2, fb[2], 1); SB();                                                                            \
-        RD_B(fb[2], P, 2, 2); ST_B(0, LWB, P); ST_B(1, LWB, P); SB();                                     \
-        RD_A(P, 3, 1); RD_B(fx[0], P, 3, 0); RD_B(fx[1], P, 3, 1); RD_B(fx[2], P, 3, 2); SB();            \
-        MM(0, fb[0], 0); SB();                                                                            \
-        ST_B(2, LWB, P); SB();                                                                            \
-        MM(1, fb[1], 0); MM(2, fb[2], 0); SB();                                                           \
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                                   \
-        RD_A((P) ^ 1, 0, 0); RD_B(fb[0], (P) ^ 1, 0, 0); RD_B(fb[1], (P) ^ 1, 0, 1);                      \
-        RD_B(fb[2], (P) ^ 1, 0, 2); SB();                                                                 \
-        MM(0, fx[0], 1); MM(1, fx[1], 1); MM(2, fx[2], 1); SB();                                          \
-    } while (0)
-#else
 #define MV_A(I, LWA, LFA, P, KTF) do { ST_A(I, LWA, P); LD_A(I, LFA, KTF); } while (0)
 #define MV_B(I, LWB, LFB, P, KTF) do { ST_B(I, LWB, P); LD_B(I, LFB, KTF); } while (0)
 #define RF_STEP(P, LWA, LWB, LFA, LFB, KTF)                                                               \
@@ -290,7 +244,6 @@ __device__ __forceinline__ void gemm_run_fast(const GemmArgs& g, f32x16 (&acc)[T
         RD_B(fb[2], (P) ^ 1, 0, 2); SB();                                                                 \
         MM(0, fx[0], 1); MM(1, fx[1], 1); MM(2, fx[2], 1); SB();                                          \
     } while (0)
-#endif
 
     la0.template load_fast_slice<0, 1, CLAMP>(A, g.a_row, g.a_k, row0, K0_OF(0), tid, g.n);
     lb0.template load_fast_slice<0, 1, CLAMP>(B, g.b_row, g.b_k, col0, K0_OF(0), tid, g.m);
@@ -520,15 +473,12 @@ __device__ __forceinline__ void gemm_store_block(const GemmArgs& g, const f32x16
 
 // Work item -> origin of its C tile: ids are regrouped so that the items of one XCD (id mod
 // 8) cover a contiguous range of tiles, then walked in groups of 8 tile-rows.
-#ifndef PTJ_GEMM_GROUP
-#define PTJ_GEMM_GROUP 8
-#endif
 __device__ __forceinline__ void tile_origin(int pid, int total, int num_m, int num_n, int& row0, int& col0) {
     {
         const int chunk = total >> 3, rem = total & 7, x = pid & 7;
         pid = x * chunk + (x < rem ? x : rem) + (pid >> 3);
     }
-    constexpr int GROUP = PTJ_GEMM_GROUP;
+    constexpr int GROUP = 8;
     const int width = GROUP * num_n;
     const int group_id = pid / width;
     const int first_m = group_id * GROUP;
@@ -736,10 +686,8 @@ __device__ __forceinline__ void gemm_stream(const GemmArgs& g, char* __restrict_
 #undef ST_B
 #undef LD_A
 #undef LD_B
-#if !PTJ_GEMM_EARLY_LOADS
 #undef MV_A
 #undef MV_B
-#endif
 
 // Persistent kernel: workgroup b handles work items b, b + gridDim.x, ... where an item is
 // one (C tile, K split) pair; the stores of a finished tile drain while the next tile's

@@ -205,14 +205,8 @@ __global__ __launch_bounds__(RowGeom<TPR>::BLOCK) void dropout_add_layernorm_ker
 // Partials layout: part[p][0][cols] = sum dy*xhat, part[p][1][cols] = sum dy over the
 // rows handled by row-slot p (p = blockIdx.x*RPB + sub).
 // ---------------------------------------------------------------------------------
-#ifndef PTJ_LN_BLOCK
-#define PTJ_LN_BLOCK 512
-#endif
-#ifndef PTJ_LN_MINW
-#define PTJ_LN_MINW 4
-#endif
 template <int TPR> struct LnBwdGeom {
-    static constexpr int BLOCK = TPR == 64 ? PTJ_LN_BLOCK : TPR;
+    static constexpr int BLOCK = TPR == 64 ? 512 : TPR;
     static constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
 };
 constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave holds (bf16, ITERS 4)
@@ -221,7 +215,7 @@ constexpr int LN_BWD_MAX_WAVE_COLS = 64 * 4 * 8;  // widest row a single wave ho
 // Philox generator out of the register budget of the common variants: 0 = no second
 // output, 1 = mask read from recorded keep bytes, 2 = mask recomputed (or eval scaling).
 template <typename T, int VEC, int TPR, int ITERS, bool DX, bool DGB, int DROP>
-__global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK, (TPR == 64 && ITERS <= 3 && DROP != 2) ? PTJ_LN_MINW : 2) void layernorm_bwd_kernel(
+__global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK, (TPR == 64 && ITERS <= 3 && DROP != 2) ? 4 : 2) void layernorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
     T* __restrict__ dx, float* __restrict__ part, int64_t rows, int cols, int64_t dys, int64_t xs, int64_t dxs,
     T* __restrict__ drop, int drop_train, uint64_t drop_seed, const uint8_t* __restrict__ keep, int np,
@@ -400,6 +394,156 @@ __global__ __launch_bounds__(LnBwdGeom<TPR>::BLOCK, (TPR == 64 && ITERS <= 3 && 
                 }
             }
         }
+    }
+}
+
+// layernorm_bwd_kernel<T, VEC, 64, ITERS, true, true, DROP> (DROP 0 or 1) for rows of exactly
+// 64 * VEC * ITERS columns: every lane holds whole vectors, so nothing is masked, and the row after
+// the current one is requested -- all of its vectors at once, in storage form -- before the current
+// row's arithmetic starts (the general kernel's loads end up interleaved with the conversions that
+// consume them, a row at a time).  Same operations in the same order as the general kernel: the
+// results are bit-equal to it.
+template <typename T, int VEC, int ITERS, int DROP>
+__global__ __launch_bounds__(512, DROP == 1 ? 2 : 4) void layernorm_bwd_exact_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ res,
+    T* __restrict__ dx, float* __restrict__ part, int64_t rows, int64_t dys, int64_t xs, int64_t dxs,
+    T* __restrict__ drop, int drop_train, const uint8_t* __restrict__ keep, int np, int has_res, int64_t ress) {
+    constexpr int TPR = 64, RPB = 8;
+    constexpr int cols = TPR * VEC * ITERS;
+    static_assert(DROP == 0 || DROP == 1, "keep-byte or no dropout output");
+    static_assert(DROP == 0 || (VEC == 4 || VEC == 8), "one keep byte per 8 columns");
+    const int t = threadIdx.x & 63;
+    const int sub = threadIdx.x >> 6;
+    Pack<T, VEC> graw[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) graw[it] = *reinterpret_cast<const Pack<T, VEC>*>(gamma + (t + it * TPR) * VEC);
+    float acc_g[ITERS][VEC], acc_b[ITERS][VEC], acc_d[ITERS][VEC];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc_g[it][j] = acc_b[it][j] = acc_d[it][j] = 0.f;
+    const float inv_n = 1.0f / (float)cols;
+    const float inv_nm1 = 1.0f / (float)(cols - 1);
+    const float n_adj = (float)cols * inv_nm1;
+    const int64_t stride = (int64_t)gridDim.x * RPB;
+    Pack<T, VEC> nx[ITERS], nd[ITERS], nr[ITERS];
+    uint8_t nk[ITERS];
+#define LNX_REQUEST(ROW)                                                                                  \
+    do {                                                                                                  \
+        const T* xr__ = x + (ROW) * xs;                                                                   \
+        const T* dr__ = dy + (ROW) * dys;                                                                 \
+        const T* rr__ = res + (ROW) * ress;                                                               \
+        _Pragma("unroll") for (int it = 0; it < ITERS; ++it) {                                            \
+            const int c__ = (t + it * TPR) * VEC;                                                         \
+            nx[it] = *reinterpret_cast<const Pack<T, VEC>*>(xr__ + c__);                                  \
+            nd[it] = *reinterpret_cast<const Pack<T, VEC>*>(dr__ + c__);                                  \
+            nr[it] = *reinterpret_cast<const Pack<T, VEC>*>(rr__ + c__);                                  \
+            if constexpr (DROP == 1) nk[it] = keep[(ROW) * (int64_t)(cols >> 3) + (c__ >> 3)];            \
+        }                                                                                                 \
+    } while (0)
+    int64_t row = (int64_t)blockIdx.x * RPB + sub;
+    if (row < rows) LNX_REQUEST(row);
+#pragma unroll 1
+    for (; row < rows; row += stride) {
+        float xv[ITERS][VEC], dv[ITERS][VEC];
+        Pack<T, VEC> rr[ITERS];
+        uint32_t kbits[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                xv[it][j] = to_f32(nx[it].v[j]);
+                dv[it][j] = to_f32(nd[it].v[j]);
+            }
+            rr[it] = nr[it];
+            if constexpr (DROP == 1) kbits[it] = (uint32_t)nk[it] >> (((t + it * TPR) * VEC) & 7);
+        }
+        // the next row of this slot (the last one asks for its own row again: no branch around the loads)
+        const int64_t nrow = row + stride < rows ? row + stride : row;
+        LNX_REQUEST(nrow);
+        __builtin_amdgcn_sched_barrier(0);
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += xv[it][j];
+        const float mu = wave_sum(s) * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float c = xv[it][j] - mu;
+                xv[it][j] = c;
+                q += c * c;
+            }
+        const float var = wave_sum(q) * inv_nm1;
+        const float rstd = 1.0f / sqrtf(var);
+        float sg = 0.f, sgx = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xh = xv[it][j] * rstd;
+                xv[it][j] = xh;
+                acc_g[it][j] += dv[it][j] * xh;
+                acc_b[it][j] += dv[it][j];
+                const float gg = dv[it][j] * to_f32(graw[it].v[j]);
+                dv[it][j] = gg;
+                sg += gg;
+                sgx += gg * xh;
+            }
+        const float mg = wave_sum(sg) * inv_n;
+        const float mgx = wave_sum(sgx) * inv_n * n_adj;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) dv[it][j] = (dv[it][j] - mg - xv[it][j] * mgx) * rstd;
+        if (has_res) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) dv[it][j] = to_f32(rr[it].v[j]) + to_f32(from_f32<T>(dv[it][j]));
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) store_vec<T, VEC>(dx + row * dxs + (t + it * TPR) * VEC, dv[it]);
+        if constexpr (DROP == 1) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const float r = to_f32(from_f32<T>(dv[it][j]));
+                    dv[it][j] = drop_train ? (((kbits[it] >> j) & 1u) ? r : 0.f) : r * 0.9f;
+                    if (np == 3) acc_d[it][j] += to_f32(from_f32<T>(dv[it][j]));   // the stored value
+                }
+                store_vec<T, VEC>(drop + row * (int64_t)cols + (t + it * TPR) * VEC, dv[it]);
+            }
+        }
+    }
+#undef LNX_REQUEST
+    // one partial per workgroup: the eight row slots are folded through LDS in slot order
+    float* pg = part + (int64_t)blockIdx.x * np * (int64_t)cols;
+    float* pb = pg + cols;
+    float* pd = pb + cols;
+    __shared__ float red[3][cols];
+    for (int sl = 0; sl < RPB; ++sl) {
+        if (sub == sl) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int c = (t + it * TPR) * VEC + j;
+                    red[0][c] = sl == 0 ? acc_g[it][j] : red[0][c] + acc_g[it][j];
+                    red[1][c] = sl == 0 ? acc_b[it][j] : red[1][c] + acc_b[it][j];
+                    red[2][c] = sl == 0 ? acc_d[it][j] : red[2][c] + acc_d[it][j];
+                }
+        }
+        __syncthreads();
+    }
+    for (int c = threadIdx.x; c < cols; c += 512) {
+        pg[c] = red[0][c];
+        pb[c] = red[1][c];
+        if (np == 3) pd[c] = red[2][c];
     }
 }
 
@@ -1021,7 +1165,17 @@ int layernorm_bwd_impl(const void* dy, const void* x, const void* gamma, const v
     // need a quarter fewer registers than two 16-byte vectors (one more wave per SIMD)
     bool launched = false;
     if constexpr (sizeof(T) == 2) {
-        if (cfg.vec == 8 && cfg.tpr == 64 && cols > 512 && cols <= 768) {
+        if (cfg.vec == 8 && cfg.tpr == 64 && cols == 768 && want_dx && want_dgb && drop_mode != 2) {
+            // whole vectors in every lane: the pipelined kernel (bit-equal to the general one)
+#define LAUNCH_X(DROP_)                                                                                           \
+    hipLaunchKernelGGL((layernorm_bwd_exact_kernel<T, 4, 3, DROP_>), dim3(grid), dim3(512), 0, st, (const T*)dy,  \
+                       (const T*)x, (const T*)gamma, (const T*)(res ? res : dy), (T*)dx, (float*)ws, rows, dys,   \
+                       xs, dxs, (T*)drop, drop_train, (const uint8_t*)keep, np, res ? 1 : 0, res ? cols : dys)
+            if (drop_mode == 0) LAUNCH_X(0);
+            else LAUNCH_X(1);
+#undef LAUNCH_X
+            launched = true;
+        } else if (cfg.vec == 8 && cfg.tpr == 64 && cols > 512 && cols <= 768) {
             LAUNCH(T, 4, 64, 3);
             launched = true;
         }

@@ -268,13 +268,17 @@ def layernorm_bkwd2_t(dloss_dx: torch.Tensor, layer_params, x: torch.Tensor, res
     return dx, (dg, db)
 
 
-def colsum_t(x: torch.Tensor):
+def colsum_t(x: torch.Tensor, out=None):
     """Sum over all leading dimensions: the bias gradient `.sum(dim=0)` of the reference's
-    t_linear_bkwd2_p (model_triton.py:426), deterministic."""
+    t_linear_bkwd2_p (model_triton.py:426), deterministic.  `out`, if given, is a contiguous
+    tensor of `cols` elements that receives the sums."""
     require_gpu(x)
     x2 = _rows2d(x)
     rows, cols = x2.shape
-    out = torch.empty(cols, dtype=x2.dtype, device=x2.device)
+    if out is None:
+        out = torch.empty(cols, dtype=x2.dtype, device=x2.device)
+    else:
+        assert out.numel() == cols and out.dtype == x2.dtype and out.is_contiguous()
     ws_bytes = lib().ptj_colsum_workspace_bytes(rows, cols)
     ws = _workspace(ws_bytes, x2.device, "colsum")
     check(lib().ptj_colsum(ptr(x2), ptr(out), ptr(ws), ws_bytes, rows, cols, x2.stride(0), dtype_code(x2), stream()),
@@ -804,8 +808,11 @@ def gpt2_bkwd_below_head_t(dh, dwemb, dbemb, acts, params, y, y_mask, train, p_g
         dsum = res[3] if i > 0 else None
     d = dropped                                                         # [N,D] = dropout_bkwd(dx, seed 0)
     # positional table: sum over the batch (model_triton.py:2518 with indices = arange(T))
-    dpos = torch.zeros_like(params[1][0])
-    dpos[:T] = colsum_t(d.view(B, T * D)).view(T, D)
+    table_rows = params[1][0].shape[0]
+    dpos = torch.empty_like(params[1][0])
+    colsum_t(d.view(B, T * D), out=dpos[:T])                            # the sums land in the table gradient itself
+    if T < table_rows:
+        dpos[T:].zero_()
     # embedding: scatter-add rows by token id, times sqrt(D); tied with the LM head (:2591)
     dwemb = embed_bkwd_add_t(dwemb, d, y)
     return [[dwemb, dbemb], [dpos]] + layer_grads + [[dlnfg, dlnfb]]
