@@ -43,6 +43,11 @@ extern "C" {
 
 int ptj_version(void);
 const char* ptj_last_error(void);
+/* Optional, once per GPU with that GPU current: resolves the per-device state that entry points
+ * otherwise look up on their first call there (the CU count that sizes the persistent grids, the
+ * device address of ptj_colsum_static's built-in scratch array), so that from the first compute
+ * call on nothing but kernel launches happens.  No counterpart in the reference. */
+int ptj_init(void);
 
 /* ---- row-wise kernels ---------------------------------------------------- */
 
@@ -97,7 +102,9 @@ int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes
  * the library (PTJ_COLSUM_STATIC_SCRATCH_BYTES per GPU, held until the process ends); shapes
  * whose partial sums do not fit -- ptj_colsum_workspace_bytes(rows, cols) above that size --
  * are rejected with PTJ_ERR_INVALID and nothing is launched.  No hipMalloc, hipFree or other
- * allocating call is made.  The GPU that `stream` belongs to must be the current device.
+ * allocating call is made; the array's device address is looked up on the first call on a GPU
+ * unless ptj_init() has done so before (callers under graph capture call ptj_init first).
+ * The GPU that `stream` belongs to must be the current device.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
  * streams, two threads) race; calls ordered on one stream are safe.  Results are bit-equal
  * to ptj_colsum's. */

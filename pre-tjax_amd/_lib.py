@@ -21,6 +21,7 @@ _p, _i64, _int, _sz = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t
 SIGNATURES = {
     "ptj_version": (_int, []),
     "ptj_last_error": (_c.c_char_p, []),
+    "ptj_init": (_int, []),
     "ptj_layernorm_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _p]),
     "ptj_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "ptj_layernorm_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _i64, _i64, _i64, _i64, _int, _p]),

@@ -1,6 +1,8 @@
 // Library-level entry points: version and thread-local error string.
 #include "common.h"
 
+#include <atomic>
+
 static thread_local char g_err[512] = "";
 
 int ptj_set_error(int code, const char* fmt, ...) {
@@ -16,21 +18,21 @@ int ptj_set_error(int code, const char* fmt, ...) {
 // has none) the MI355X's 256.
 int ptj_num_cus() {
     constexpr int DEFAULT_CUS = 256, MAX_DEVICES = 64;
-    static int cached[MAX_DEVICES] = {};
+    static std::atomic<int> cached[MAX_DEVICES] = {};   // 0 = not asked yet; every thread that asks stores the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
         (void)hipGetLastError();
         return DEFAULT_CUS;
     }
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
             (void)hipGetLastError();
             n = DEFAULT_CUS;
         }
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 extern "C" {

@@ -24,7 +24,14 @@ __device__ __forceinline__ void ce_load_to_lds(const void* gsrc, void* lds_wave_
 // vector stores that were issued AFTER them may still be in flight (vector memory operations
 // of one wavefront complete in issue order, so "all but the newest N" covers the copies).
 // `younger` is wave-uniform; anything outside 0..8 waits for everything.
+// The count is exact only while every gradient vector of a row is ONE store instruction
+// (ce_exact_store_count says for which wavefronts that is so); a count that is too high would read
+// a landing area that has not filled yet.  CE_RELAXED_ROW_WAIT = false takes that assumption out
+// (every wait then drains the stores too): measured 0.79 against 0.76 ms for the 16384 x 50257 pass.
+// The parity tests against the CPU oracle and against the plain pass run with the relaxed wait.
+constexpr bool CE_RELAXED_ROW_WAIT = true;
 __device__ __forceinline__ void ce_wait_row_landed(int younger) {
+    if (!CE_RELAXED_ROW_WAIT) younger = -1;
     switch (younger) {
         case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
         case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;

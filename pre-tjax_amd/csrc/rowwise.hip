@@ -1398,6 +1398,16 @@ int ptj_colsum(const void* x, void* out, void* workspace, size_t workspace_bytes
                  (colsum_impl<bf16>(x, out, workspace, workspace_bytes, rows, cols, xs, st)));
 }
 
+int ptj_init(void) {
+    // per-device state that entry points otherwise look up on their first call: the address of
+    // the built-in scratch array and the CU count
+    void* ws = nullptr;
+    const int rc = colsum_static_scratch(&ws);
+    if (rc != PTJ_OK) return rc;
+    (void)ptj_num_cus();
+    return PTJ_OK;
+}
+
 int ptj_colsum_static(const void* x, void* out, int64_t rows, int64_t cols, int64_t xs, int dtype, void* stream) {
     PTJ_CHECK_ARG(rows >= 1 && cols >= 1 && cols < (1ll << 31), "colsum_static: bad shape");
     PTJ_CHECK_ARG(x && out, "colsum_static: null pointer");

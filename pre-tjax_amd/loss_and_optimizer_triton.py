@@ -34,8 +34,10 @@ def t_avg_cross_entropy_loss_bkwd3_t(y_labels: torch.Tensor, x_logits: torch.Ten
     count = torch.empty((), dtype=torch.int64, device=x2.device)
     if inplace:
         dx = x2
-    else:  # same row pitch as the logits, so rows keep their 16-byte phase
-        dx = torch.empty_strided((rows, cols), (x2.stride(0), 1), dtype=x2.dtype, device=x2.device)
+    else:  # same row pitch and the same offset inside a 16-byte line as the logits, so rows keep their phase
+        mis = (x2.data_ptr() % 16) // x2.element_size()
+        flat = torch.empty((rows - 1) * x2.stride(0) + cols + mis, dtype=x2.dtype, device=x2.device)
+        dx = flat[mis:].as_strided((rows, cols), (x2.stride(0), 1))
     pred = torch.empty(rows, dtype=torch.int64, device=x2.device) if want_pred else None
     colsum = None
     fused = (want_colsum and x2.dtype == torch.bfloat16 and x2.stride(0) % 8 == 0 and dx.stride(0) % 8 == 0

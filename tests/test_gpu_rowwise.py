@@ -197,6 +197,53 @@ def test_ce_with_column_sums_equals_separate_passes(lo, mt, rows, V, pitch):
     assert torch.equal(loss2, loss0)
 
 
+@pytest.mark.parametrize("shift,inplace", [(3, False), (3, True), (5, True), (8, False)])
+def test_ce_with_column_sums_rows_off_the_16_byte_grid(lo, mt, shift, inplace):
+    """Logits whose rows start `shift` elements into 16-byte aligned, 8-element-pitched rows (a column
+    slice of a wider buffer): the vectors that hold a row's two ends are stored element by element
+    and the partial column sums are indexed by slot.  Against the plain pass and the fp64 sums."""
+    rows, V, pitch = 300, 4099, 4112
+    g = gen(67 + shift)
+    buf = randn(g, rows, pitch, dtype=torch.bfloat16).to(DEV)
+    x = buf[:, shift:shift + V]
+    assert (x.data_ptr() % 16 != 0) == (shift % 8 != 0)
+    y = torch.randint(0, V, (rows,), generator=g)
+    y[::4] = 0
+    y = y.to(DEV)
+    loss0, cnt0, dx0, pred0 = lo.t_avg_cross_entropy_loss_bkwd3_t(y, x, want_pred=True)
+    wl, wc, wdx = ops.avg_cross_entropy_loss_bkwd3(y.cpu(), f64(x))
+    assert abs(loss0.item() - wl.item()) <= 1e-4 * abs(wl.item())
+    assert_close(dx0, wdx, torch.bfloat16, atol=1e-6, what="ce dlogits (shifted rows)")
+    xin = buf.clone()[:, shift:shift + V] if inplace else x
+    keep_left, keep_right = buf[:, :shift].clone(), buf[:, shift + V:].clone()
+    loss1, cnt1, dx1, pred1, sums = lo.t_avg_cross_entropy_loss_bkwd3_t(y, xin, inplace=inplace, want_pred=True,
+                                                                     want_colsum=True)
+    assert torch.equal(loss0, loss1) and torch.equal(cnt0, cnt1) and torch.equal(pred0, pred1) and torch.equal(dx0, dx1)
+    if inplace:
+        assert dx1.data_ptr() == xin.data_ptr()
+    want = f64(dx1).sum(0)
+    assert ((f64(sums) - want).abs() <= 2 ** -8 * want.abs() + 1e-9).all()
+    # nothing outside the rows was written
+    if not inplace:
+        assert torch.equal(buf[:, :shift], keep_left) and torch.equal(buf[:, shift + V:], keep_right)
+
+
+@pytest.mark.parametrize("dtype,pitch", [(torch.float32, 1000), (torch.bfloat16, 1003)])
+def test_ce_column_sums_where_the_fused_pass_does_not_apply(lo, mt, dtype, pitch):
+    """fp32 logits, or a row pitch that is not a multiple of 8: want_colsum routes to the plain pass
+    plus colsum_t and returns the same values as the two calls made by hand."""
+    rows, V = 130, 1000
+    g = gen(68)
+    x = randn(g, rows, pitch, dtype=dtype).to(DEV)[:, :V]
+    y = torch.randint(0, V, (rows,), generator=g).to(DEV)
+    loss0, cnt0, dx0 = lo.t_avg_cross_entropy_loss_bkwd3_t(y, x)
+    loss1, cnt1, dx1, sums = lo.t_avg_cross_entropy_loss_bkwd3_t(y, x, want_colsum=True)
+    assert torch.equal(loss0, loss1) and torch.equal(dx0, dx1) and torch.equal(sums, mt.colsum_t(dx0))
+    want = f64(dx0).sum(0)
+    tol = 1e-5 if dtype == torch.float32 else 2 ** -8
+    assert ((f64(sums) - want).abs() <= tol * want.abs() + 1e-9).all()
+
+
 def test_ce_all_labels_zero_is_nan(lo):
     x = torch.randn(4, 50, device=DEV)
     loss, cnt, dx = lo.t_avg_cross_entropy_loss_bkwd3_t(torch.zeros(4, dtype=torch.int64, device=DEV), x)

@@ -25,6 +25,25 @@ def _both(l, x, rows, cols, stride, code, stream):
     return out_ws, out_st
 
 
+def test_colsum_static_after_init_takes_no_device_memory():
+    """With ptj_init() done, a ptj_colsum_static call changes neither the free device memory nor
+    torch's allocator state (inputs and output are allocated before the measurement)."""
+    _lib = importlib.import_module("pre-tjax_amd._lib")
+    l = _lib.lib()
+    assert l.ptj_init() == 0, l.ptj_last_error()
+    rows, cols = 2048, 768
+    x = torch.randn(rows, cols, device=DEV)
+    out = torch.empty(cols, device=DEV)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    stats0 = torch.cuda.memory_stats()["allocation.all.allocated"]
+    assert l.ptj_colsum_static(x.data_ptr(), out.data_ptr(), rows, cols, cols, 0, torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_stats()["allocation.all.allocated"] == stats0
+    assert torch.allclose(out.double(), x.double().sum(0), rtol=1e-5, atol=1e-3)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_colsum_static_equals_colsum_twice_second_call_smaller(dtype):
     _lib = importlib.import_module("pre-tjax_amd._lib")
