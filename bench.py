@@ -105,8 +105,10 @@ def attn_leg(torch, mt, B, H, T, dh, dtype, train, mask_tensor=False):
     q, k, v = qkv.unbind(2)
     mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=dev)).expand(B, T, T).contiguous() if mask_tensor else None
     o, ms_, ls_ = mt.attn_fwd_t(q, k, v, mask, train, 5)
-    t_af = _timeit(torch, lambda: mt.attn_fwd_t(q, k, v, mask, train, 5))
-    t_ab = _timeit(torch, lambda: mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, mask, train, 5))
+    # long warm-ups: the clocks of an idle chip take tens of milliseconds to settle, which would
+    # otherwise favour whichever leg runs later
+    t_af = _timeit(torch, lambda: mt.attn_fwd_t(q, k, v, mask, train, 5), n=40, warm=200)
+    t_ab = _timeit(torch, lambda: mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, mask, train, 5), n=40, warm=100)
     causal = dh * B * H * T * (T + 1) // 2
     peak = PEAK_BF16_TFLOPS if dtype == torch.bfloat16 else PEAK_FP32_TFLOPS
     tot = 14 * causal / ((t_af + t_ab) * 1e-3) / 1e12
@@ -233,9 +235,10 @@ def only_leg(torch, mt, lo, which, c):
         qkv = torch.randn(B, H, 3, T, dh, device=dev).to(bf)
         dO = torch.randn(B, H, T, dh, device=dev).to(bf)
         q, k, v = qkv.unbind(2)
+        mask = torch.tril(torch.ones(T, T, dtype=torch.bool, device=dev)).expand(B, T, T).contiguous()
         for _ in range(3):
-            o, ms_, ls_ = mt.attn_fwd_t(q, k, v, None, True, 5)
-            mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, None, True, 5)
+            o, ms_, ls_ = mt.attn_fwd_t(q, k, v, mask, True, 5)
+            mt.attn_bwd_t(dO, q, k, v, o, ms_, ls_, mask, True, 5)
     elif which == "gemm":
         x = torch.randn(N, D, device=dev).to(bf)
         w1 = torch.randn(F, D, device=dev).to(bf)
@@ -244,6 +247,18 @@ def only_leg(torch, mt, lo, which, c):
             mt.matmul_t(x, w1.t())          # forward product   [N,D] x [D,F]   (both operands K-major)
             mt.matmul_t(dy, w1)             # dX product        [N,F] x [F,D]   (B transposed on load)
             mt.matmul_t(dy.t(), x)          # dW product        [F,N] x [N,D]   (both transposed, K split)
+    elif which == "rowwise":
+        # the step's LayerNorm launches, each over 12 buffer sets (more than the last-level cache holds)
+        xs_ = [torch.randn(N, D, device=dev).to(bf) for _ in range(12)]
+        dys = [torch.randn(N, D, device=dev).to(bf) for _ in range(12)]
+        rss = [torch.randn(N, D, device=dev).to(bf) for _ in range(12)]
+        gam = torch.ones(D, device=dev, dtype=bf)
+        keeps = [mt.dropout_add_t(xs_[i], rss[i], True, 42, want_keep=True)[1] for i in range(12)]
+        for i in range(12):
+            mt.t_layernorm_fwd_t((gam, gam), xs_[i])
+            mt.dropout_add_layernorm_t(xs_[i], rss[i], (gam, gam), True, 42, want_keep=True)
+            mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i])
+            mt.layernorm_bkwd2_t(dys[i], (gam, gam), xs_[i], residual=rss[i], drop=(True, 42, keeps[i]), drop_sum=True)
     else:
         logits = mt._padded_logits(N, V, bf, dev)
         lab = torch.randint(0, V, (N,), device=dev)
@@ -251,7 +266,7 @@ def only_leg(torch, mt, lo, which, c):
             logits.normal_()
             lo.t_avg_cross_entropy_loss_bkwd3_t(lab, logits, inplace=True, want_pred=True, want_colsum=True)
     torch.cuda.synchronize()
-    print(json.dumps({"only": which, "launch_sets": 3}))
+    print(json.dumps({"only": which, "launch_sets": 12 if which == "rowwise" else 3}))
 
 
 def main():
@@ -263,7 +278,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the legs of baseline configurations 2, 3 and 4")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run one plain 1 GiB device copy first (reference reading for FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--only", choices=["attn", "gemm", "ce"], default=None,
+    ap.add_argument("--only", choices=["attn", "gemm", "ce", "rowwise"], default=None,
                     help="run just a few launches of one kernel family at the step's shapes and exit "
                          "(short programs for rocprofv3 counter passes)")
     ap.add_argument("--steps-only", action="store_true",
@@ -285,6 +300,12 @@ def main():
     c = CFG
     B, T, V = c["B"], c["T"], c["V"]
 
+    if args.copy_probe:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.only is not None:
         only_leg(torch, mt, lo, args.only, c)
         return
@@ -307,12 +328,6 @@ def main():
         lo.adam_w_in_place(master, grads, 6e-4, (0.9, 0.95), 1e-8, moments, i, 0.1, wd_mask, shadow=shadow)
         losses.append(loss)
 
-    if args.copy_probe:
-        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
