@@ -251,7 +251,7 @@ def test_ce_all_labels_zero_is_nan(lo):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(4096, 768), (33, 200), (7, 2048), (3, 5000)])
+@pytest.mark.parametrize("shape", [(4096, 768), (1000, 768), (37, 768), (33, 200), (7, 2048), (3, 5000)])
 def test_layernorm_bwd_with_dropout_output_matches_separate_calls(mt, dtype, shape):
     """The LayerNorm backward that also emits dropout_bkwd(dx): bit-exact against the
     LayerNorm backward followed by the dropout kernel, train and eval."""
