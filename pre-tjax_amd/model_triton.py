@@ -443,15 +443,46 @@ def _bhr(t):
     return t.stride(0), t.stride(1), t.stride(2)
 
 
+ATTN_DH = 64   # head dimension of the attention kernels
+
+
+def _pad_heads(t, scale=None):
+    """[..., dh] -> [..., 64] with zero columns (optionally times `scale`): zero columns add
+    nothing to q.k and produce zero output columns."""
+    out = torch.zeros(t.shape[:-1] + (ATTN_DH,), dtype=t.dtype, device=t.device)
+    out[..., :t.shape[-1]] = t if scale is None else t * scale
+    return out
+
+
+def _aligned_view(t):
+    """Kernel operand requirements: 16-byte aligned base, strides multiple of 16 bytes."""
+    vec = 16 // t.element_size()
+    if t.stride(3) != 1 or t.data_ptr() % 16 or any(s % vec for s in t.stride()[:3]):
+        return t.contiguous()
+    return t
+
+
 def attn_fwd_t(q, k, v, mask, train, seed, out=None):
     """Flash-attention forward on [B,H,T,dh] *views* (any batch/head/row strides).
-    Returns (O, ms[B,H,T] fp32, ls[B,H,T] fp32).  `out` may be a preallocated view."""
+    Returns (O, ms[B,H,T] fp32, ls[B,H,T] fp32).  `out` may be a preallocated view.
+
+    The kernels are written for dh = 64.  Smaller head sizes (the reference takes any power of
+    two, model_triton.py:716) are run on zero-padded copies: q is scaled by sqrt(64/dh) so that
+    the kernels' 1/sqrt(64) gives 1/sqrt(dh), and O is cut back to dh columns."""
     require_gpu(q, k, v)
     B, H, T, dh = q.shape
     assert k.shape == q.shape and v.shape == q.shape and q.dtype == k.dtype == v.dtype
     assert T % 64 == 0, "sequence length must be a multiple of 64"
+    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
+    if dh < ATTN_DH:
+        o, ms, ls = attn_fwd_t(_pad_heads(q, math.sqrt(ATTN_DH / dh)), _pad_heads(k), _pad_heads(v), mask, train, seed)
+        if out is None:
+            return o[..., :dh].contiguous(), ms, ls
+        out.copy_(o[..., :dh])
+        return out, ms, ls
     if out is None:
         out = torch.empty((B, H, T, dh), dtype=q.dtype, device=q.device)
+    q, k, v = _aligned_view(q), _aligned_view(k), _aligned_view(v)
     ms = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
     ls = torch.empty_like(ms)
     m = _mask_arg(mask, B, T)
@@ -465,12 +496,25 @@ def attn_fwd_t(q, k, v, mask, train, seed, out=None):
 
 def attn_bwd_t(d_o, q, k, v, o, ms, ls, mask, train, seed, out=None):
     """Flash-attention backward on [B,H,T,dh] views; returns (dq, dk, dv) (views of `out`
-    = (dq, dk, dv) when given)."""
+    = (dq, dk, dv) when given).  Head sizes below 64 run on zero-padded copies as in the forward
+    (q' = f q with f = sqrt(64/dh), so dq = f dq')."""
     require_gpu(d_o, q, k, v, o)
     B, H, T, dh = q.shape
+    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
+    if dh < ATTN_DH:
+        f = math.sqrt(ATTN_DH / dh)
+        dq, dk, dv = attn_bwd_t(_pad_heads(d_o), _pad_heads(q, f), _pad_heads(k), _pad_heads(v), _pad_heads(o), ms, ls,
+                                mask, train, seed)
+        if out is None:
+            return dq[..., :dh] * f, dk[..., :dh].contiguous(), dv[..., :dh].contiguous()
+        out[0].copy_(dq[..., :dh] * f)
+        out[1].copy_(dk[..., :dh])
+        out[2].copy_(dv[..., :dh])
+        return out
     if out is None:
         out = tuple(torch.empty((B, H, T, dh), dtype=q.dtype, device=q.device) for _ in range(3))
     dq, dk, dv = out
+    d_o, q, k, v, o = (_aligned_view(t) for t in (d_o, q, k, v, o))
     m = _mask_arg(mask, B, T)
     ws_bytes = lib().ptj_attn_workspace_bytes(B, H, T)
     ws = _workspace(ws_bytes, q.device, "attn")
@@ -483,59 +527,20 @@ def attn_bwd_t(d_o, q, k, v, o, ms, ls, mask, train, seed, out=None):
     return dq, dk, dv
 
 
-def _aligned_view(t):
-    """Kernel operand requirements: 16-byte aligned base, strides multiple of 16 bytes."""
-    vec = 16 // t.element_size()
-    if t.stride(3) != 1 or t.data_ptr() % 16 or any(s % vec for s in t.stride()[:3]):
-        return t.contiguous()
-    return t
-
-
-ATTN_DH = 64   # head dimension of the attention kernels
-
-
-def _pad_heads(t, scale=None):
-    """[..., dh] -> [..., 64] with zero columns (optionally times `scale`): zero columns add
-    nothing to q.k and produce zero output columns."""
-    out = torch.zeros(t.shape[:-1] + (ATTN_DH,), dtype=t.dtype, device=t.device)
-    out[..., :t.shape[-1]] = t if scale is None else t * scale
-    return out
-
-
 def t_scaled_dot_prod_attn_fwd3_t(qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
-    """qkv [B,H,3,T,dh], mask [B,T,T] bool -> (O [B,H,T,dh], [ms, ls, O]).
-
-    The kernels are written for dh = 64.  Smaller head sizes (the reference takes any power of
-    two, model_triton.py:716) are run on zero-padded copies: q is scaled by sqrt(64/dh) so that
-    the kernels' 1/sqrt(64) gives 1/sqrt(dh), and O is cut back to dh columns."""
+    """qkv [B,H,3,T,dh], mask [B,T,T] bool -> (O [B,H,T,dh], [ms, ls, O]) (model_triton.py:706-754)."""
     if train:
         assert p_gen_aux is not None
-    dh = qkv.shape[-1]
-    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
     q, k, v = torch.unbind(qkv, dim=2)
-    if dh < ATTN_DH:
-        o, ms, ls = attn_fwd_t(_pad_heads(q, math.sqrt(ATTN_DH / dh)), _pad_heads(k), _pad_heads(v), mask, train,
-                               p_gen_aux)
-        o = o[..., :dh].contiguous()
-        return o, [ms, ls, o]
-    o, ms, ls = attn_fwd_t(_aligned_view(q), _aligned_view(k), _aligned_view(v), mask, train, p_gen_aux)
+    o, ms, ls = attn_fwd_t(q, k, v, mask, train, p_gen_aux)
     return o, [ms, ls, o]
 
 
 def t_scaled_dot_prod_attn_bkwd3_t(dloss_dx, acts, qkv: torch.Tensor, mask: torch.Tensor, train=True, p_gen_aux=None):
-    """-> (dq, dk, dv), each [B,H,T,dh]."""
+    """-> (dq, dk, dv), each [B,H,T,dh] (model_triton.py:951-1003)."""
     ms, ls, o = acts
-    dh = qkv.shape[-1]
-    assert dh <= ATTN_DH, "head dimension %d > %d is not supported" % (dh, ATTN_DH)
     q, k, v = torch.unbind(qkv, dim=2)
-    if dh < ATTN_DH:
-        f = math.sqrt(ATTN_DH / dh)
-        dq, dk, dv = attn_bwd_t(_pad_heads(dloss_dx), _pad_heads(q, f), _pad_heads(k), _pad_heads(v), _pad_heads(o), ms,
-                                ls, mask, train, p_gen_aux)
-        # q' = f q: dq = f dq'
-        return dq[..., :dh] * f, dk[..., :dh].contiguous(), dv[..., :dh].contiguous()
-    return attn_bwd_t(_aligned_view(dloss_dx), _aligned_view(q), _aligned_view(k), _aligned_view(v), _aligned_view(o), ms,
-                      ls, mask, train, p_gen_aux)
+    return attn_bwd_t(dloss_dx, q, k, v, o, ms, ls, mask, train, p_gen_aux)
 
 
 def _masked_scores(q, k, mask):

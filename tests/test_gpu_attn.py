@@ -316,8 +316,14 @@ def test_attn_rejects_bad_shapes(mt):
     qkv = torch.zeros(1, 1, 3, 96, 64, device=DEV)
     with pytest.raises(AssertionError):
         mt.t_scaled_dot_prod_attn_fwd3_t(qkv, None, False)
+    # the C ABI itself takes dh = 64 only (the wrappers pad smaller heads)
     q = torch.zeros(1, 1, 64, 32, device=DEV)
-    with pytest.raises(_lib.PtjError):
-        mt.attn_fwd_t(q, q, q, None, False, 0)               # the C ABI itself takes dh = 64 only
+    o, ms = torch.empty_like(q), torch.empty(1, 1, 64, device=DEV)
+    st = (q.stride(0), q.stride(1), q.stride(2))
+    rc = _lib.lib().ptj_attn_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), None, o.data_ptr(), ms.data_ptr(), ms.data_ptr(),
+                                 None, 0, 1, 1, 64, 32, *st, *st, *st, *st, 0, 0, _lib.PTJ_F32, _lib.stream())
+    assert rc != 0 and b"head dimension" in _lib.lib().ptj_last_error()
+    o2, _, _ = mt.attn_fwd_t(q, q, q, None, False, 0)
+    assert o2.shape == q.shape
     with pytest.raises(AssertionError):
         mt.t_scaled_dot_prod_attn_fwd3_t(torch.zeros(1, 1, 3, 64, 128, device=DEV), None, False)

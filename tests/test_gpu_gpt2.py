@@ -63,6 +63,21 @@ def test_small_model_grads(lo, dtype, train, mask_as):
         assert abs(acc.item() - wacc.item()) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("train", [False, True])
+def test_small_model_grads_head_size_32(lo, dtype, train):
+    """Head size 32 (the reference's two-layer test model, tests/test_fwd3_t.ipynb cell 0: D64, H2)
+    through the composite forward and backward: the attention wrappers run it on zero-padded heads."""
+    grads, loss, acc, frac, want_g, wl, wacc, wfrac = run_case(lo, V=128, D=64, L=2, H=2, F=256, T=128, B=2,
+                                                               dtype=dtype, train=train, seed=7)
+    ltol, gtol = (1e-5, 5e-5) if dtype == torch.float32 else (5e-3, 2e-2)
+    assert abs(loss.item() - wl.item()) <= ltol * abs(wl.item()), (loss.item(), wl.item())
+    for gi, (gg, wg) in enumerate(zip(grads, want_g)):
+        for pi, (a, b) in enumerate(zip(gg, wg)):
+            assert a.shape == b.shape, (gi, pi, a.shape, b.shape)
+            assert rel_l2(a, b) <= gtol, "grad[%d][%d] rel L2 %.3e" % (gi, pi, rel_l2(a, b))
+
+
 def test_gpt2_small_config1_fp32(lo):
     # BASELINE config 1: full GPT-2 small, fp32, B=2, T=256, dropout off (eval semantics, x0.9)
     grads, loss, acc, frac, want_g, wl, wacc, wfrac = run_case(lo, V=50257, D=768, L=12, H=12, F=3072, T=256, B=2,
